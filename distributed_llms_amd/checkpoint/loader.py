@@ -32,13 +32,13 @@ def load_tokenizer(model_path: str):
 def load_model(model_id: str, device_map: str = "auto", dtype: Optional[str] = None) -> Tuple[object, object]:
     """Load a checkpoint dir (HF layout or ``shards/``) or a ``synthetic:<preset>`` into one stage."""
     from ..config import get_model_config, resolve_device, torch_dtype
-    from ..models.stage import ModelStage
+    from ..models import make_stage
     from .shard_manager import iter_checkpoint
 
     dev = resolve_device("auto" if device_map in (None, "auto") else device_map)
     dt = torch_dtype(dtype or ("bfloat16" if dev.startswith("cuda") else "float32"))
     cfg = get_model_config(model_id)
-    stage = ModelStage(cfg, 0, cfg.num_layers, device=dev, dtype=dt)
+    stage = make_stage(cfg, 0, cfg.num_layers, device=dev, dtype=dt)
     if model_id.startswith("synthetic:") or not os.path.isdir(model_id):
         stage.init_synthetic(0)
         return stage, None

@@ -16,13 +16,13 @@ import dataclasses
 import json
 import os
 from dataclasses import dataclass, field
-from typing import Any, Dict, Optional
+from typing import Any, Dict, List, Optional
 
 
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2"
+    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2", "tudilix" (layer-list hybrid)
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -39,8 +39,23 @@ class ModelConfig:
     experts_per_token: int = 0     # MoE top-k
     bos_token_id: int = 1
     eos_token_id: int = 2
+    # layer-list models (arch "tudilix"): one entry per layer, {"type": "attention" | "rglru",
+    # "mixer": {...sizes and constants of the mixer...}, "mlp": {...} | None}; every size of such a
+    # model is read from its entry (the flat fields above hold the widest layer, for planning only)
+    layers: Optional[List[Dict[str, Any]]] = None
+    residual_mult: float = 1.0     # sublayer outputs enter the residual stream scaled by this
+    logit_softcap: float = 0.0     # > 0: logits <- cap * tanh(logits / cap)
 
     # ------------------------------------------------------------------ sizes
+    @property
+    def is_layer_list(self) -> bool:
+        return self.layers is not None
+
+    @property
+    def needs_state_slots(self) -> bool:
+        """Sequences carry per-layer state besides paged K/V (recurrent state, convolution tails)."""
+        return self.layers is not None
+
     @property
     def q_size(self) -> int:
         return self.num_heads * self.head_dim
@@ -59,6 +74,9 @@ class ModelConfig:
 
     def layer_param_count(self) -> int:
         h, i = self.hidden_size, self.intermediate_size
+        if self.layers is not None:
+            from .models.hybrid import layer_param_count
+            return sum(layer_param_count(h, l) for l in self.layers) // max(1, len(self.layers))
         attn = h * self.qkv_size + self.q_size * h
         if self.arch == "gpt2":
             attn += self.qkv_size + h  # biases
@@ -88,11 +106,19 @@ class ModelConfig:
                 + self.head_param_count())
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
+        if self.layers is not None:
+            from .models.hybrid import kv_width
+            return sum(kv_width(l) for l in self.layers) * dtype_bytes
         return 2 * self.num_layers * self.kv_size * dtype_bytes
 
     # ----------------------------------------------------------- HF interop
     def to_hf_config(self) -> Dict[str, Any]:
         """A ``config.json``-compatible dict (written into ``shards/config.json``)."""
+        if self.layers is not None:
+            return {"architecture": "Tudilix", "layers": [dict(l) for l in self.layers],
+                    "logit_softcap": self.logit_softcap, "norm": {"eps": self.norm_eps},
+                    "residual_mult": self.residual_mult, "vocab": self.vocab_size, "width": self.hidden_size,
+                    "_dllm_name": self.name}
         if self.arch == "gpt2":
             return {
                 "model_type": "gpt2", "architectures": ["GPT2LMHeadModel"],
@@ -124,6 +150,8 @@ class ModelConfig:
 
     @staticmethod
     def from_hf_config(cfg: Dict[str, Any], name: Optional[str] = None) -> "ModelConfig":
+        if cfg.get("architecture") == "Tudilix":
+            return ModelConfig.from_layer_list(cfg, name)
         mt = cfg.get("model_type", "llama")
         name = name or cfg.get("_dllm_name") or cfg.get("_name_or_path") or mt
         eos = cfg.get("eos_token_id", 2)
@@ -155,6 +183,31 @@ class ModelConfig:
             num_experts=cfg.get("num_local_experts", 0) if mt == "mixtral" else 0,
             experts_per_token=cfg.get("num_experts_per_tok", 0) if mt == "mixtral" else 0,
             bos_token_id=cfg.get("bos_token_id", 1), eos_token_id=eos)
+
+
+def _from_layer_list(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelConfig:
+    """A layer-list ``config.json`` ("architecture": "Tudilix"): keys ``layers`` (per layer ``type``,
+    ``mixer``, ``mlp``), ``width``, ``vocab``, ``norm.eps``, ``residual_mult``, ``logit_softcap``."""
+    layers = [dict(l) for l in cfg["layers"]]
+    if not layers:
+        raise ValueError("layer-list config without layers")
+    attn = [l["mixer"] for l in layers if l["type"] == "attention"]
+    for l in layers:
+        if l["type"] not in ("attention", "rglru"):
+            raise ValueError(f"unsupported layer type {l['type']!r} (attention, rglru)")
+        if l.get("mlp") is not None and l["mlp"].get("kind", "dense") != "dense":
+            raise ValueError(f"unsupported mlp kind {l['mlp'].get('kind')!r} (dense)")
+    ff = max([l["mlp"]["ff"] for l in layers if l.get("mlp")] or [0])
+    return ModelConfig(
+        name=name or cfg.get("_dllm_name") or "tudilix", arch="tudilix", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), intermediate_size=int(ff), num_layers=len(layers),
+        num_heads=max([m["heads"] for m in attn] or [1]), num_kv_heads=max([m["kv_heads"] for m in attn] or [1]),
+        head_dim=max([max(m["dim"], m["vdim"]) for m in attn] or [1]), max_position=1 << 30,
+        norm_eps=float(cfg["norm"]["eps"]), bos_token_id=-1, eos_token_id=-1, layers=layers,
+        residual_mult=float(cfg.get("residual_mult", 1.0)), logit_softcap=float(cfg.get("logit_softcap", 0.0)))
+
+
+ModelConfig.from_layer_list = staticmethod(_from_layer_list)
 
 
 _LLAMA3_ROPE = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
@@ -196,6 +249,25 @@ PRESETS: Dict[str, ModelConfig] = {
         intermediate_size=384, num_layers=4, num_heads=4, num_kv_heads=2, head_dim=64,
         max_position=1024, rope_theta=1000000.0, norm_eps=1e-5,
         num_experts=4, experts_per_token=2, bos_token_id=1, eos_token_id=2),
+    "tiny-tudilix": _from_layer_list({
+        "architecture": "Tudilix", "vocab": 384, "width": 128, "residual_mult": 0.7, "logit_softcap": 20.0,
+        "norm": {"eps": 1e-6},
+        "layers": [
+            {"type": "rglru", "mixer": {"blocks": 2, "conv": 4, "width": 192}, "mlp": None},
+            {"type": "attention", "mixer": {
+                "conv": 3, "dim": 32, "vdim": 48, "heads": 4, "kv_heads": 2, "mask": {"size": 40}, "scale": 0.2,
+                "rot": {"base": 10000.0, "dims": 24,
+                        "scaling": {"factor": 8.0, "fast": 16.0, "original": 512, "slow": 2.0}}},
+             "mlp": {"kind": "dense", "ff": 320, "limit": 2.0}},
+            {"type": "rglru", "mixer": {"blocks": 3, "conv": 2, "width": 192},
+             "mlp": {"kind": "dense", "ff": 192, "limit": 1.5}},
+            {"type": "attention", "mixer": {
+                "conv": 2, "dim": 32, "vdim": 48, "heads": 4, "kv_heads": 2, "kv_from": 1, "mask": {"size": 17},
+                "scale": 0.15,
+                "rot": {"base": 10000.0, "dims": 24,
+                        "scaling": {"factor": 8.0, "fast": 16.0, "original": 512, "slow": 2.0}}},
+             "mlp": None},
+        ]}, name="tiny-tudilix"),
     "tiny-gpt2": ModelConfig(
         name="tiny-gpt2", arch="gpt2", vocab_size=512, hidden_size=128,
         intermediate_size=512, num_layers=4, num_heads=2, num_kv_heads=2, head_dim=64,

@@ -13,7 +13,7 @@
 
 void register_block_manager(py::module_& m) {
   py::class_<BlockManager>(m, "BlockManager")
-      .def(py::init<int, int>(), py::arg("num_blocks"), py::arg("block_size"))
+      .def(py::init<int, int, int>(), py::arg("num_blocks"), py::arg("block_size"), py::arg("num_state_slots") = 0)
       .def_property_readonly("num_blocks", &BlockManager::num_blocks)
       .def_property_readonly("block_size", &BlockManager::block_size)
       .def("num_free", &BlockManager::num_free)
@@ -28,5 +28,9 @@ void register_block_manager(py::module_& m) {
       .def("block_table", &BlockManager::block_table)
       .def("fill_block_tables", &BlockManager::fill_block_tables, py::arg("seqs"), py::arg("out"),
            py::arg("pad") = 0)
-      .def("fill_slots", &BlockManager::fill_slots);
+      .def("fill_slots", &BlockManager::fill_slots)
+      .def_property_readonly("num_state_slots", &BlockManager::num_state_slots)
+      .def("num_free_state_slots", &BlockManager::num_free_state_slots)
+      .def("state_slot", &BlockManager::state_slot)
+      .def("fill_state_slots", &BlockManager::fill_state_slots);
 }

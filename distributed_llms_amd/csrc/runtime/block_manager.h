@@ -16,16 +16,41 @@ namespace py = pybind11;
 
 class BlockManager {
  public:
-  BlockManager(int num_blocks, int block_size) : num_blocks_(num_blocks), block_size_(block_size) {
+  // `num_state_slots` > 0: every sequence also owns one fixed-size STATE SLOT from its first block
+  // to free_sequence() -- the row of the per-layer state pools (recurrent state, the inputs a
+  // short causal convolution still needs) of models whose layers carry state besides paged K/V.
+  // 0: no state slots (attention-only models).
+  BlockManager(int num_blocks, int block_size, int num_state_slots = 0)
+      : num_blocks_(num_blocks), block_size_(block_size), num_state_slots_(num_state_slots) {
     if (num_blocks <= 0 || block_size <= 0) throw std::invalid_argument("num_blocks/block_size must be > 0");
+    if (num_state_slots < 0) throw std::invalid_argument("num_state_slots must be >= 0");
     free_.reserve(num_blocks);
     for (int b = num_blocks - 1; b >= 0; --b) free_.push_back(b);
+    for (int s = num_state_slots - 1; s >= 0; --s) free_states_.push_back(s);
   }
 
   int num_blocks() const { return num_blocks_; }
   int block_size() const { return block_size_; }
   int num_free() const { return (int)free_.size(); }
   int num_sequences() const { return (int)tables_.size(); }
+  int num_state_slots() const { return num_state_slots_; }
+  int num_free_state_slots() const { return (int)free_states_.size(); }
+
+  // The sequence's state slot; -1 without state slots, throws for an unknown sequence.
+  int32_t state_slot(int64_t seq) const {
+    if (!num_state_slots_) return -1;
+    auto it = states_.find(seq);
+    if (it == states_.end()) throw std::out_of_range("sequence has no state slot");
+    return it->second;
+  }
+
+  void fill_state_slots(py::array_t<int64_t, py::array::c_style> seqs,
+                        py::array_t<int32_t, py::array::c_style> out) const {
+    auto s = seqs.unchecked<1>();
+    auto o = out.mutable_unchecked<1>();
+    if (o.shape(0) < s.shape(0)) throw std::invalid_argument("state slot buffer too small");
+    for (py::ssize_t i = 0; i < s.shape(0); ++i) o(i) = state_slot(s(i));
+  }
   int blocks_for(int64_t tokens) const { return (int)((tokens + block_size_ - 1) / block_size_); }
 
   bool has_sequence(int64_t seq) const { return tables_.count(seq) != 0; }
@@ -49,6 +74,11 @@ class BlockManager {
   bool ensure_capacity(int64_t seq, int64_t tokens) {
     const int need = extra_blocks_needed(seq, tokens);
     if (need > num_free()) return false;
+    if (num_state_slots_ && !states_.count(seq)) {
+      if (free_states_.empty()) return false;
+      states_[seq] = free_states_.back();
+      free_states_.pop_back();
+    }
     auto& t = tables_[seq];
     for (int i = 0; i < need; ++i) {
       t.push_back(free_.back());
@@ -71,6 +101,11 @@ class BlockManager {
   }
 
   void free_sequence(int64_t seq) {
+    auto st = states_.find(seq);
+    if (st != states_.end()) {
+      free_states_.push_back(st->second);
+      states_.erase(st);
+    }
     auto it = tables_.find(seq);
     if (it == tables_.end()) return;
     for (auto b = it->second.rbegin(); b != it->second.rend(); ++b) free_.push_back(*b);
@@ -128,5 +163,8 @@ class BlockManager {
   int block_size_;
   std::vector<int32_t> free_;
   std::unordered_map<int64_t, std::vector<int32_t>> tables_;
+  int num_state_slots_;
+  std::vector<int32_t> free_states_;
+  std::unordered_map<int64_t, int32_t> states_;
 };
 

@@ -36,6 +36,8 @@ class HostBatch:
     # mixed prefill + decode step: the first num_decode sequences are single-token decode rows
     # (decode attention), the rest prefill chunks (prefill attention); 0 = not mixed
     num_decode: int = 0
+    # [B] int32 state slot of every sequence (models with per-sequence state besides K/V), else None
+    state_slots: Optional[np.ndarray] = None
     # the packed array this batch was unpacked from (its fields are views into it): pack() then
     # only refreshes the header instead of concatenating everything again
     raw: Optional[np.ndarray] = field(default=None, repr=False, compare=False)
@@ -58,12 +60,15 @@ class HostBatch:
         b, t = self.num_seqs, self.num_tokens
         mb = self.block_tables.shape[1] if self.block_tables.ndim == 2 else 0
         has_s = 1 if self.sampling is not None else 0
+        has_st = 1 if self.state_slots is not None else 0
         hdr = np.array([1 if self.is_prefill else 0, t, b, mb, self.max_q_len, self.max_ctx, self.slot,
-                        self.step_id, has_s, self.num_decode] + [0] * 6, dtype=np.int32)
+                        self.step_id, has_s, self.num_decode, has_st] + [0] * 5, dtype=np.int32)
         parts = [hdr, self.ids, self.positions, self.slots, self.seq_lens, self.cu_seqlens,
                  self.block_tables.reshape(-1), self.logits_idx]
         if has_s:
             parts.append(self.sampling.reshape(-1))
+        if has_st:
+            parts.append(self.state_slots)
         return np.concatenate([p.astype(np.int32, copy=False).reshape(-1) for p in parts])
 
     def sampling_args(self) -> dict:
@@ -76,7 +81,7 @@ class HostBatch:
     @staticmethod
     def unpack(arr: np.ndarray) -> "HostBatch":
         hdr = arr[:16]
-        pf, t, b, mb, mq, mc, slot, sid, has_s, nd = (int(x) for x in hdr[:10])
+        pf, t, b, mb, mq, mc, slot, sid, has_s, nd, has_st = (int(x) for x in hdr[:11])
         o = 16
         def take(n):
             nonlocal o
@@ -88,8 +93,9 @@ class HostBatch:
         bt = take(b * mb).reshape(b, mb)
         lidx = take(b)
         samp = take(3 * b).reshape(b, 3) if has_s else None
+        states = take(b) if has_st else None
         return HostBatch(bool(pf), ids, pos, slots, seq_lens, cu, bt, lidx, mq, mc, slot, sid, samp, raw=arr,
-                         num_decode=nd)
+                         num_decode=nd, state_slots=states)
 
 
 def next_pow2(x: int, lo: int = 1) -> int:
@@ -97,6 +103,17 @@ def next_pow2(x: int, lo: int = 1) -> int:
     while p < x:
         p *= 2
     return p
+
+
+def _with_state(hb: HostBatch, seq_ids, bm) -> HostBatch:
+    """Attach the sequences' state slots (a BlockManager that hands them out: models whose layers
+    keep recurrent / convolution state per sequence)."""
+    if getattr(bm, "num_state_slots", 0):
+        ids = np.ascontiguousarray(seq_ids, dtype=np.int64)
+        hb.state_slots = np.empty(ids.shape[0], dtype=np.int32)
+        bm.fill_state_slots(ids, hb.state_slots)
+        hb.raw = None
+    return hb
 
 
 def build_host_batch(step: Step, bm, block_size: int, max_blocks: Optional[int] = None,
@@ -107,10 +124,13 @@ def build_host_batch(step: Step, bm, block_size: int, max_blocks: Optional[int] 
     if getattr(step, "mixed", False):
         dec = HostBatch.unpack(step.packed)
         pre = build_host_batch(Step(True, step.seqs, step.slot), bm, block_size, None, step_id)
-        return merge_mixed(dec, pre, step.slot, step_id)
+        pre.state_slots = None
+        ids = np.concatenate([np.asarray(step.rows, dtype=np.int64),
+                              np.fromiter((s.seq_id for s in step.seqs), dtype=np.int64)])
+        return _with_state(merge_mixed(dec, pre, step.slot, step_id), ids, bm)
     if step.packed is not None:
         step.packed[7] = step_id
-        return HostBatch.unpack(step.packed)
+        return _with_state(HostBatch.unpack(step.packed), step.rows, bm)
     seqs = step.seqs
     b = len(seqs)
     seq_ids = np.fromiter((s.seq_id for s in seqs), dtype=np.int64, count=b)
@@ -156,8 +176,8 @@ def build_host_batch(step: Step, bm, block_size: int, max_blocks: Optional[int] 
     if any(s.params.temperature > 0 for s in seqs):
         sampling = np.array([[int(round(s.params.temperature * 1e4)), int(s.params.top_k),
                               int(round(s.params.top_p * 1e4))] for s in seqs], dtype=np.int32)
-    return HostBatch(step.is_prefill, ids, positions, slots, seq_lens, cu, bt, logits_idx, max_q_len,
-                     max_ctx, step.slot, step_id, sampling)
+    return _with_state(HostBatch(step.is_prefill, ids, positions, slots, seq_lens, cu, bt, logits_idx, max_q_len,
+                                 max_ctx, step.slot, step_id, sampling), seq_ids, bm)
 
 
 def merge_mixed(dec: HostBatch, pre: HostBatch, slot: int, step_id: int) -> HostBatch:
@@ -198,9 +218,9 @@ def build_decode_batch(seq_ids: np.ndarray, seq_lens: np.ndarray, bm, block_size
         raise ValueError("max_blocks too small for batch")
     bt = np.zeros((b, max_blocks), dtype=np.int32)
     bm.fill_block_tables(seq_ids, bt, 0)
-    return HostBatch(False, np.zeros(b, dtype=np.int32), positions, slots, seq_lens.astype(np.int32),
-                     np.arange(b + 1, dtype=np.int32), bt, np.arange(b, dtype=np.int32), 1,
-                     int(seq_lens.max()) if b else 0, slot, step_id, None)
+    return _with_state(HostBatch(False, np.zeros(b, dtype=np.int32), positions, slots, seq_lens.astype(np.int32),
+                                 np.arange(b + 1, dtype=np.int32), bt, np.arange(b, dtype=np.int32), 1,
+                                 int(seq_lens.max()) if b else 0, slot, step_id, None), seq_ids, bm)
 
 
 def to_device_meta(hb: HostBatch, device, pad_ctx_to: Optional[int] = None) -> (torch.Tensor, BatchMeta):
@@ -220,6 +240,11 @@ def to_device_meta(hb: HostBatch, device, pad_ctx_to: Optional[int] = None) -> (
         logits_idx=up(hb.logits_idx, torch.int64) if hb.is_prefill else None,
         max_q_len=hb.max_q_len, max_ctx=pad_ctx_to or hb.max_ctx, num_seqs=hb.num_seqs,
         num_tokens=hb.num_tokens)
+    if hb.state_slots is not None:
+        meta.state_slots = up(hb.state_slots)
+        meta.tok_seq = up(np.repeat(np.arange(hb.num_seqs, dtype=np.int32), np.diff(hb.cu_seqlens)))
+        if meta.cu_seqlens_q is None:
+            meta.cu_seqlens_q = up(hb.cu_seqlens)
     nd = hb.num_decode
     if nd and hb.is_prefill:
         # mixed step: the prefill rows' own cu_seqlens (from 0) and the decode rows' context bound

@@ -17,6 +17,7 @@ import torch
 
 from .. import _ext, knobs
 from ..config import EngineConfig, resolve_device, torch_dtype
+from ..models import make_stage
 from ..models.stage import ModelStage
 from .batch import build_host_batch
 from .graphs import SCRATCH_SEQ_ID
@@ -28,9 +29,9 @@ from .sequence import SamplingParams, Sequence
 log = logging.getLogger("dllm.engine")
 
 
-def make_block_manager(num_blocks: int, block_size: int):
-    bm = _ext.runtime().BlockManager(num_blocks, block_size)
-    # block 0 is the scratch block padded decode rows write into
+def make_block_manager(num_blocks: int, block_size: int, num_state_slots: int = 0):
+    bm = _ext.runtime().BlockManager(num_blocks, block_size, num_state_slots)
+    # block 0 (and state slot 0) is the scratch block padded decode rows write into
     assert bm.ensure_capacity(SCRATCH_SEQ_ID, 1)
     assert bm.block_table(SCRATCH_SEQ_ID) == [0]
     return bm
@@ -44,7 +45,7 @@ def build_stage(ecfg: EngineConfig, layer_start: int = 0, layer_end: Optional[in
     layer_end = mcfg.num_layers if layer_end is None else layer_end
     dev = resolve_device(device or ecfg.device)
     dtype = torch_dtype(ecfg.dtype)
-    stage = ModelStage(mcfg, layer_start, layer_end, device=dev, dtype=dtype, units=units, tp=tp,
+    stage = make_stage(mcfg, layer_start, layer_end, device=dev, dtype=dtype, units=units, tp=tp,
                        unit_group=unit_group)
     if shard_state is not None:
         stage.load_hf_state(shard_state)
@@ -70,7 +71,7 @@ class LLMEngine:
             ecfg = self.ecfg = ecfg.apply_overrides(use_graphs=False, streams=1)
         self.num_slots = max(1, ecfg.streams) if gpu else 1
         self.runner = StageRunner(self.stage, ecfg, num_slots=self.num_slots)
-        self.bm = make_block_manager(self.runner.num_blocks, ecfg.kv_block_size)
+        self.bm = make_block_manager(self.runner.num_blocks, ecfg.kv_block_size, self.runner.num_state_slots)
         # max_batch is the engine's total decode batch, split evenly over the slots
         per_slot = -(-ecfg.max_batch // self.num_slots)
         self.scheduler = Scheduler(self.bm, self.num_slots, per_slot, ecfg.max_prefill_tokens, ecfg.max_seq_len,

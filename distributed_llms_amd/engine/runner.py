@@ -20,9 +20,10 @@ log = logging.getLogger("dllm.runner")
 
 
 def plan_kv_blocks(mcfg: ModelConfig, num_layers: int, ecfg: EngineConfig, device,
-                   num_kv_heads: Optional[int] = None) -> int:
+                   num_kv_heads: Optional[int] = None, bytes_per_block: int = 0) -> int:
     """KV blocks for a stage: enough for max_batch x max_seq_len (+ scratch), capped by free HBM.
-    ``num_kv_heads``: the heads this rank caches (its share under tensor parallelism)."""
+    ``num_kv_heads``: the heads this rank caches (its share under tensor parallelism);
+    ``bytes_per_block``: the stage's own figure (layers whose caches differ in shape)."""
     bs = ecfg.kv_block_size
     if ecfg.num_kv_blocks > 0:
         return ecfg.num_kv_blocks
@@ -30,7 +31,8 @@ def plan_kv_blocks(mcfg: ModelConfig, num_layers: int, ecfg: EngineConfig, devic
     # microbatch slots in flight (the pipeline driver's, config.pipeline_slots)
     slots = pipeline_slots(ecfg, ecfg.num_workers, device)
     want = ecfg.max_batch * slots * per_seq + 2
-    per_block = max(1, KVCache.bytes_per_block(num_layers, num_kv_heads or mcfg.num_kv_heads, mcfg.head_dim, bs))
+    per_block = max(1, bytes_per_block or
+                    KVCache.bytes_per_block(num_layers, num_kv_heads or mcfg.num_kv_heads, mcfg.head_dim, bs))
     dev = torch.device(device)
     if dev.type == "cuda":
         free, _total = torch.cuda.mem_get_info(dev)
@@ -58,13 +60,22 @@ class StageRunner:
         if ecfg.kernel_knobs:
             knobs.update(ecfg.kernel_knobs)
         self.block_size = ecfg.kv_block_size
-        nb = num_blocks or plan_kv_blocks(stage.cfg, stage.num_layers, ecfg, stage.device, stage.hkv)
+        own = stage.kv_bytes_per_block(self.block_size) if hasattr(stage, "kv_bytes_per_block") else 0
+        nb = num_blocks or plan_kv_blocks(stage.cfg, stage.num_layers, ecfg, stage.device, stage.hkv, own)
         stage.allocate_kv(nb, self.block_size)
         self.num_blocks = nb
+        # state slots (models with recurrent / convolution state per sequence): one per sequence that
+        # can be live on any microbatch slot, plus slot 0, the scratch sequence's
+        self.num_state_slots = 0
+        if stage.cfg.needs_state_slots:
+            self.num_state_slots = ecfg.max_batch * pipeline_slots(ecfg, ecfg.num_workers, stage.device) + 1
+            stage.allocate_state(self.num_state_slots)
         self.max_blocks = -(-ecfg.max_seq_len // self.block_size)
         self._busy = None                 # [(start, end) events or host seconds] while metering
         self.graph_sets = []
-        if ecfg.use_graphs and stage.device.type == "cuda":
+        # decode graphs replay fixed buffers of the attention-only step; steps of models with state
+        # slots launch eagerly
+        if ecfg.use_graphs and stage.device.type == "cuda" and not stage.cfg.needs_state_slots:
             sizes = [b for b in ecfg.graph_batch_sizes if b <= ecfg.max_batch] or [ecfg.max_batch]
             if max(sizes) < ecfg.max_batch:
                 sizes.append(ecfg.max_batch)

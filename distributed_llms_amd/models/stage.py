@@ -54,6 +54,10 @@ class BatchMeta:
     cu_seqlens_p: Optional[torch.Tensor] = None
     max_ctx_d: int = 0
     max_q_len_p: int = 0
+    # models with per-sequence state besides K/V (BlockManager state slots): the sequences' slots [B]
+    # and each token's sequence index [T]; cu_seqlens_q is then set for decode steps too
+    state_slots: Optional[torch.Tensor] = None
+    tok_seq: Optional[torch.Tensor] = None
 
 
 class KVCache:

@@ -1,0 +1,392 @@
+"""Ops of layer-list models whose layers carry per-sequence state: a float32 residual stream with
+pre- and post-sublayer RMS norms, short causal convolutions with a state tail, the real-gated linear
+recurrent unit (RG-LRU), sliding-window attention over a paged K/V cache whose key and value widths
+differ, a clipped GLU and the logit soft cap.
+
+Same dispatch as :mod:`distributed_llms_amd.ops`: a CUDA tensor goes to the in-tree HIP kernels
+(csrc/kernels/seqmix.hip, attention_window.hip) and raises if they are not built; CPU tensors run
+the plain PyTorch forms below (the ``_ref_*`` functions).  Activations (``act``) are bfloat16 or
+float32; what feeds a norm, a softmax, a rotation angle, a gate of the recurrence or the recurrent
+state itself is float32 in both.
+
+Varlen batches: a step's tokens are the concatenation of B sequence chunks, ``cu`` [B + 1] their
+offsets, ``positions`` [T] each token's position in its sequence, ``tok_seq`` [T] its chunk,
+``state_slots`` [B] the row of every state pool the sequence owns.  A chunk that starts at position
+0 starts from zero state (its slot's previous content is never read).
+"""
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Optional, Tuple
+
+import torch
+
+from .. import _ext
+
+ACT_DTYPES = (torch.bfloat16, torch.float32)
+
+
+@dataclass
+class SeqBatch:
+    """Device-side varlen metadata of one step (a view of the stage's BatchMeta)."""
+    cu: torch.Tensor            # [B + 1] int32
+    positions: torch.Tensor     # [T] int32
+    tok_seq: torch.Tensor       # [T] int32
+    state_slots: torch.Tensor   # [B] int32
+    num_seqs: int
+    num_tokens: int
+    max_q_len: int
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _k():
+    return _ext.kernels()
+
+
+def _f32flag(t: torch.Tensor) -> int:
+    if t.dtype not in ACT_DTYPES:
+        raise TypeError(f"activation dtype {t.dtype} (bfloat16 or float32)")
+    return 1 if t.dtype == torch.float32 else 0
+
+
+def _ck(t: torch.Tensor, name: str, dtype=None):
+    if dtype is not None and t.dtype != dtype:
+        raise TypeError(f"{name}: expected {dtype}, got {t.dtype}")
+    if not t.is_contiguous():
+        raise ValueError(f"{name}: must be contiguous")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+# ------------------------------------------------------------------ embedding / norms
+def embedding_f32(ids: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """Rows of ``table`` as a float32 residual stream [T, W]."""
+    if not table.is_cuda:
+        return table.index_select(0, ids.long()).float()
+    _ck(ids, "ids", torch.int32)
+    _ck(table, "table")
+    t, (v, w) = ids.numel(), table.shape
+    out = torch.empty(t, w, dtype=torch.float32, device=table.device)
+    _k().sm_embed_f32(out.data_ptr(), ids.data_ptr(), table.data_ptr(), t, w, v, _f32flag(table), _stream())
+    return out
+
+
+def _ref_rms(x: torch.Tensor, w: torch.Tensor, eps: float, offset: float) -> torch.Tensor:
+    x = x.float()
+    return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + eps) * (offset + w.float())
+
+
+def rms_norm_f32(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype, one_plus: bool = True) -> torch.Tensor:
+    """x [T, W] float32 -> x / sqrt(mean(x^2) + eps) * ((1 if one_plus else 0) + w) in ``act_dtype``."""
+    if not x.is_cuda:
+        return _ref_rms(x, w, eps, 1.0 if one_plus else 0.0).to(act_dtype)
+    _ck(x, "x", torch.float32)
+    _ck(w, "w", act_dtype)
+    t, width = x.shape
+    y = torch.empty(t, width, dtype=act_dtype, device=x.device)
+    _k().sm_rms_norm(y.data_ptr(), x.data_ptr(), w.data_ptr(), t, width, float(eps), 1.0 if one_plus else 0.0,
+                     _f32flag(y), _stream())
+    return y
+
+
+def post_norm_add(x: torch.Tensor, o: torch.Tensor, w_post: torch.Tensor, eps: float, mult: float,
+                  bias: Optional[torch.Tensor] = None, w_next: Optional[torch.Tensor] = None):
+    """The close of a sublayer, fused: ``x += mult * rms_norm(o + bias) * (1 + w_post)`` in place on the
+    float32 residual stream; with ``w_next`` also returns the next sublayer's input
+    ``rms_norm(x) * (1 + w_next)`` in ``o``'s dtype (None otherwise)."""
+    if not x.is_cuda:
+        ob = o.float() if bias is None else o.float() + bias.float()
+        x.add_(mult * _ref_rms(ob, w_post, eps, 1.0))
+        return x, (None if w_next is None else _ref_rms(x, w_next, eps, 1.0).to(o.dtype))
+    _ck(x, "x", torch.float32)
+    _ck(o, "o")
+    t, width = x.shape
+    if o.shape != x.shape:
+        raise ValueError("post_norm_add: o / x shape mismatch")
+    h = torch.empty_like(o) if w_next is not None else None
+    _k().sm_post_norm_add(x.data_ptr(), o.data_ptr(), _ptr(bias), w_post.data_ptr(), _ptr(w_next), _ptr(h), t, width,
+                          float(eps), float(mult), _f32flag(o), _stream())
+    return x, h
+
+
+# ------------------------------------------------------------------ causal convolution with state
+def _ref_conv_gather(u: torch.Tensor, state: torch.Tensor, sb: SeqBatch, taps: int,
+                     in_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """[taps, T, C] float32: tap j of token t is the input at position p_t - (taps - 1) + j (the
+    chunk's own rows, the state tail before the chunk's start, zeros before the sequence's)."""
+    t, c = u.shape
+    out = torch.zeros(taps, t, c, dtype=torch.float32, device=u.device)
+    cu = sb.cu.tolist()
+    pos = sb.positions.tolist()
+    slots = sb.state_slots.tolist()
+    for b in range(sb.num_seqs):
+        a, e = cu[b], cu[b + 1]
+        if e == a:
+            continue
+        start = pos[a]
+        prev = state[slots[b]].float() if start > 0 else torch.zeros(taps - 1, c, device=u.device)
+        if 0 < start < taps - 1:
+            prev = torch.cat([torch.zeros(taps - 1 - start, c, device=u.device), prev[taps - 1 - start:]], 0)
+        full = torch.cat([prev, u[a:e].float()], 0)
+        state[slots[b]] = full[full.shape[0] - (taps - 1):].to(state.dtype)
+        if in_bias is not None:        # added to every input that exists (not to the zeros before position 0)
+            full = full.clone()
+            full[max(0, taps - 1 - start):] += in_bias.float()
+        for j in range(taps):
+            out[j, a:e] = full[j:j + (e - a)]
+    return out
+
+
+def causal_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                sb: SeqBatch, out_dtype=torch.float32, in_bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Per-channel causal convolution over time, y_t = bias + sum_j w[:, j] (u + in_bias)_(t - taps + 1 + j)
+    (zeros before the sequence's start), across chunk borders: ``state`` [slots, taps - 1, C] holds each
+    sequence's last taps - 1 rows of ``u`` and is brought up to date.  ``u`` [T, C] may be a column slice
+    of a wider projection (row stride); ``in_bias`` is the bias of the projection that made it."""
+    c, taps = w.shape
+    if u.shape[1] != c or state.shape[1:] != (taps - 1, c):
+        raise ValueError("causal_conv: shape mismatch")
+    if not u.is_cuda:
+        g = _ref_conv_gather(u, state, sb, taps, in_bias)
+        y = (g * w.float().t()[:, None, :]).sum(0)
+        if bias is not None:
+            y = y + bias.float()
+        return y.to(out_dtype)
+    if u.stride(1) != 1:
+        raise ValueError("causal_conv: channels must be contiguous")
+    _ck(w, "w", u.dtype)
+    _ck(state, "state", u.dtype)
+    y = torch.empty(u.shape[0], c, dtype=out_dtype, device=u.device)
+    _k().sm_causal_conv(y.data_ptr(), u.data_ptr(), u.stride(0), w.data_ptr(), _ptr(bias), _ptr(in_bias), state.data_ptr(),
+                        sb.cu.data_ptr(), sb.positions.data_ptr(), sb.tok_seq.data_ptr(), sb.state_slots.data_ptr(),
+                        sb.num_tokens, sb.num_seqs, c, taps, _f32flag(u), 1 if out_dtype == torch.float32 else 0,
+                        _stream())
+    return y
+
+
+# ------------------------------------------------------------------ RG-LRU
+def gelu_tanh_f32(z: torch.Tensor) -> torch.Tensor:
+    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z * z * z)))
+
+
+def rglru(u: torch.Tensor, y_raw: torch.Tensor, y_bias: torch.Tensor, ra_t: torch.Tensor, ra_b: torch.Tensor,
+          ri_t: torch.Tensor, ri_b: torch.Tensor, lam: torch.Tensor, state: torch.Tensor, sb: SeqBatch,
+          act_dtype, decay_scale: float = 8.0) -> torch.Tensor:
+    """Real-gated linear recurrent unit over a varlen batch.
+
+    ``u`` [T, C] float32 (the convolved branch), split into ``nb`` blocks of ``bw`` channels;
+    r = sigmoid(Ra_b u_b + ra_b), i = sigmoid(Ri_b u_b + ri_b) with ``ra_t`` / ``ri_t`` [nb, bw_in, bw_out]
+    (the gate matrices TRANSPOSED, so consecutive outputs are consecutive in memory);
+    a = exp(-decay_scale * r * softplus(lam)); S_t = a S_(t-1) + sqrt(1 - a^2) * i * u, all float32,
+    ``state`` [slots, C] float32 carried between chunks.  Returns S_t * gelu_tanh(y_raw + y_bias) in
+    ``act_dtype`` (``y_raw`` [T, C], row-strided allowed)."""
+    t, c = u.shape
+    nb, bw, _ = ra_t.shape
+    if nb * bw != c:
+        raise ValueError("rglru: blocks x block width != channels")
+    if not u.is_cuda:
+        ub = u.float().view(t, nb, bw)
+        r = torch.sigmoid(torch.einsum("tbi,bio->tbo", ub, ra_t.float()).reshape(t, c) + ra_b.float().reshape(c))
+        ig = torch.sigmoid(torch.einsum("tbi,bio->tbo", ub, ri_t.float()).reshape(t, c) + ri_b.float().reshape(c))
+        a = torch.exp(-decay_scale * r * torch.nn.functional.softplus(lam.float()))
+        g = torch.sqrt(1.0 - a * a) * ig * u.float()
+        s_all = torch.empty(t, c, dtype=torch.float32)
+        cu, pos, slots = sb.cu.tolist(), sb.positions.tolist(), sb.state_slots.tolist()
+        for b in range(sb.num_seqs):
+            lo, hi = cu[b], cu[b + 1]
+            if hi == lo:
+                continue
+            s = state[slots[b]].clone() if pos[lo] > 0 else torch.zeros(c)
+            for k in range(lo, hi):
+                s = a[k] * s + g[k]
+                s_all[k] = s
+            state[slots[b]] = s
+        return (s_all * gelu_tanh_f32(y_raw.float() + y_bias.float())).to(act_dtype)
+    _ck(u, "u", torch.float32)
+    _ck(state, "state", torch.float32)
+    if y_raw.stride(1) != 1:
+        raise ValueError("rglru: y_raw channels must be contiguous")
+    for n, x in (("ra_t", ra_t), ("ri_t", ri_t), ("ra_b", ra_b), ("ri_b", ri_b), ("lam", lam), ("y_bias", y_bias)):
+        _ck(x, n, act_dtype)
+    a = torch.empty(t, c, dtype=torch.float32, device=u.device)
+    g = torch.empty(t, c, dtype=torch.float32, device=u.device)
+    f = _f32flag(y_raw)
+    _k().sm_rglru_gates(a.data_ptr(), g.data_ptr(), u.data_ptr(), ra_t.data_ptr(), ra_b.data_ptr(), ri_t.data_ptr(),
+                        ri_b.data_ptr(), lam.data_ptr(), t, nb, bw, float(decay_scale), f, _stream())
+    out = torch.empty(t, c, dtype=act_dtype, device=u.device)
+    _k().sm_rglru_scan(out.data_ptr(), a.data_ptr(), g.data_ptr(), y_raw.data_ptr(), y_raw.stride(0),
+                       y_bias.data_ptr(), state.data_ptr(), sb.cu.data_ptr(), sb.positions.data_ptr(),
+                       sb.state_slots.data_ptr(), sb.num_seqs, c, sb.max_q_len, f, _stream())
+    return out
+
+
+# ------------------------------------------------------------------ clipped GLU / soft cap
+def clipped_glu(gu: torch.Tensor, bias_gu: Optional[torch.Tensor], limit: float, alpha: float = 1.702) -> torch.Tensor:
+    """[T, 2F] = gate | up (+ bias): g = min(gate, limit), u = clamp(up, -limit, limit);
+    g * sigmoid(alpha g) * (u + 1)  -> [T, F]."""
+    t, two_f = gu.shape
+    f = two_f // 2
+    if not gu.is_cuda:
+        x = gu.float() if bias_gu is None else gu.float() + bias_gu.float()
+        g = torch.clamp(x[:, :f], max=limit)
+        u = torch.clamp(x[:, f:], -limit, limit)
+        return (g * torch.sigmoid(alpha * g) * (u + 1.0)).to(gu.dtype)
+    _ck(gu, "gu")
+    out = torch.empty(t, f, dtype=gu.dtype, device=gu.device)
+    _k().sm_clipped_glu(out.data_ptr(), gu.data_ptr(), _ptr(bias_gu), t, f, float(limit), float(alpha), _f32flag(gu),
+                        _stream())
+    return out
+
+
+def softcap_f32(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """float32 cap * tanh(logits / cap) (cap <= 0: a plain float32 copy)."""
+    if not logits.is_cuda:
+        x = logits.float()
+        return cap * torch.tanh(x / cap) if cap > 0 else x
+    _ck(logits, "logits")
+    out = torch.empty(logits.shape, dtype=torch.float32, device=logits.device)
+    _k().sm_softcap(out.data_ptr(), logits.data_ptr(), logits.numel(), float(cap), _f32flag(logits), _stream())
+    return out
+
+
+# ------------------------------------------------------------------ rotary tables
+def yarn_frequencies(dims: int, base: float, scaling: Optional[dict]) -> Tuple[torch.Tensor, float]:
+    """(f [dims / 2] float32, magnitude): rotary frequencies f_i = base^(-2i/dims), blended by YaRN
+    (``scaling``: factor, original, fast, slow): with d(t) = dims ln(original / (2 pi t)) / (2 ln base),
+    lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1), ramp_i = clamp((i - lo) / max(hi - lo,
+    0.001), 0, 1), f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i); cos and sin are scaled by
+    0.1 ln(factor) + 1."""
+    i = torch.arange(dims // 2, dtype=torch.float64)
+    f = torch.pow(torch.tensor(float(base), dtype=torch.float64), -2.0 * i / dims)
+    mag = 1.0
+    if scaling:
+        factor = float(scaling["factor"])
+
+        def d(turns):
+            return dims * math.log(scaling["original"] / (2 * math.pi * turns)) / (2 * math.log(base))
+        lo = max(math.floor(d(scaling["fast"])), 0)
+        hi = min(math.ceil(d(scaling["slow"])), dims - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0, 1)
+        f = f / factor * ramp + f * (1 - ramp)
+        mag = 0.1 * math.log(factor) + 1.0
+    return f.float(), float(mag)
+
+
+def _ref_rope_interleaved(x: torch.Tensor, pos: torch.Tensor, freqs: torch.Tensor, mag: float) -> torch.Tensor:
+    """x [T, H, D] float32; pairs (2i, 2i + 1) for i < len(freqs) rotate by pos * f_i."""
+    n = freqs.numel()
+    ang = pos.float()[:, None] * freqs.float()[None]
+    c, s = (torch.cos(ang) * mag)[:, None, :], (torch.sin(ang) * mag)[:, None, :]
+    out = x.clone()
+    a, b = x[..., 0:2 * n:2], x[..., 1:2 * n:2]
+    out[..., 0:2 * n:2] = a * c - b * s
+    out[..., 1:2 * n:2] = b * c + a * s
+    return out
+
+
+# ------------------------------------------------------------------ attention input: conv + norm + rotation + append
+def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_norm: torch.Tensor,
+              k_norm: Optional[torch.Tensor], freqs: torch.Tensor, mag: float, eps: float,
+              k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slot_mapping: torch.Tensor,
+              sb: SeqBatch, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
+    """From the fused projection [T, heads * dim (+ kv_heads * dim + kv_heads * vdim)]: the short causal
+    convolution on every channel (``conv_w`` [C, taps], tail in ``state`` [slots, taps - 1, C]), the
+    per-head RMS norm of q and k (plain weight), the interleaved-pair rotation of their first
+    2 len(freqs) dims, and the append of k [.., dim] and v [.., vdim] (convolved only) at
+    ``slot_mapping`` into caches [NB, kv_heads, BS, dim] / [NB, kv_heads, BS, vdim].  With
+    ``k_cache`` None the projection holds q only (the layer reads another layer's K/V).
+    Returns q [T, heads, dim]."""
+    t, c = qkv.shape
+    own_kv = k_cache is not None
+    qc, kc, vc = heads * dim, kv_heads * dim, kv_heads * vdim
+    if c != qc + (kc + vc if own_kv else 0) or conv_w.shape[0] != c:
+        raise ValueError("attn_prep: projection width mismatch")
+    taps = conv_w.shape[1]
+    if not qkv.is_cuda:
+        g = _ref_conv_gather(qkv, state, sb, taps)
+        y = (g * conv_w.float().t()[:, None, :]).sum(0)
+        pos = sb.positions
+        q = _ref_rms(y[:, :qc].view(t, heads, dim), q_norm, eps, 0.0)
+        q = _ref_rope_interleaved(q, pos, freqs, mag).to(qkv.dtype)
+        if own_kv:
+            k = _ref_rms(y[:, qc:qc + kc].view(t, kv_heads, dim), k_norm, eps, 0.0)
+            k = _ref_rope_interleaved(k, pos, freqs, mag)
+            v = y[:, qc + kc:].view(t, kv_heads, vdim)
+            bs = k_cache.shape[2]
+            sm = slot_mapping.long()
+            k_cache[sm // bs, :, sm % bs] = k.to(k_cache.dtype)
+            v_cache[sm // bs, :, sm % bs] = v.to(v_cache.dtype)
+        return q
+    _ck(qkv, "qkv")
+    _ck(conv_w, "conv_w", qkv.dtype)
+    _ck(state, "state", qkv.dtype)
+    _ck(freqs, "freqs", torch.float32)
+    if state.shape[1:] != (taps - 1, c):
+        raise ValueError("attn_prep: state shape")
+    if own_kv:
+        _ck(k_cache, "k_cache", qkv.dtype)
+        _ck(v_cache, "v_cache", qkv.dtype)
+        if k_cache.shape[1:] != (kv_heads, k_cache.shape[2], dim) or v_cache.shape[1:] != (kv_heads, k_cache.shape[2], vdim):
+            raise ValueError("attn_prep: cache shape")
+    if 2 * freqs.numel() > dim:
+        raise ValueError("attn_prep: rotary dims exceed the head size")
+    q = torch.empty(t, heads, dim, dtype=qkv.dtype, device=qkv.device)
+    _k().sm_attn_prep(q.data_ptr(), qkv.data_ptr(), conv_w.data_ptr(), state.data_ptr(), q_norm.data_ptr(),
+                      _ptr(k_norm), freqs.data_ptr(), freqs.numel(), float(mag), float(eps), _ptr(k_cache),
+                      _ptr(v_cache), slot_mapping.data_ptr(), sb.cu.data_ptr(), sb.positions.data_ptr(),
+                      sb.tok_seq.data_ptr(), sb.state_slots.data_ptr(), sb.num_tokens, sb.num_seqs, heads,
+                      kv_heads if own_kv else 0, dim, vdim, taps, k_cache.shape[2] if own_kv else 1,
+                      _f32flag(qkv), _stream())
+    return q
+
+
+# ------------------------------------------------------------------ sliding-window attention
+def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
+                     sb: SeqBatch, window: int, scale: float, num_decode: Optional[int] = None) -> torch.Tensor:
+    """Softmax attention of every query token over the keys j of its own sequence with
+    0 <= p - j < window (p the query's position), keys / values read through ``block_tables`` from
+    caches [NB, G, BS, dim] / [NB, G, BS, vdim]; query head h reads K/V head h // (H / G).
+    Scores and weights are float32.  ``num_decode``: the first that many sequences are one-token
+    rows (they take the decode kernel; None: every sequence is one); the rest are prompt chunks.
+    Returns [T, H, vdim]."""
+    t, h, d = q.shape
+    g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    if not q.is_cuda:
+        out = torch.empty(t, h, dv, dtype=torch.float32)
+        pos, seq = sb.positions.tolist(), sb.tok_seq.tolist()
+        rep = h // g
+        for i in range(t):
+            p = pos[i]
+            lo = max(0, p - window + 1)
+            idx = torch.arange(lo, p + 1)
+            blk = block_tables[seq[i]].long()[idx // bs]
+            kk = k_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)     # [n, H, d]
+            vv = v_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)
+            s = torch.einsum("hd,nhd->hn", q[i].float(), kk) * scale
+            out[i] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+        return out.to(q.dtype)
+    _ck(q, "q")
+    _ck(k_cache, "k_cache", q.dtype)
+    _ck(v_cache, "v_cache", q.dtype)
+    _ck(block_tables, "block_tables", torch.int32)
+    if h % g or k_cache.shape[3] != d or window < 1:
+        raise ValueError("window_attention: head / size mismatch")
+    out = torch.empty(t, h, dv, dtype=q.dtype, device=q.device)
+    nd = sb.num_seqs if num_decode is None else int(num_decode)
+    f = _f32flag(q)
+    if nd:       # one-token rows are the first nd tokens
+        _k().sm_window_attn_decode(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                   block_tables.data_ptr(), block_tables.shape[1], sb.positions.data_ptr(),
+                                   sb.tok_seq.data_ptr(), nd, h, g, d, dv, bs, int(window), float(scale), f, _stream())
+    if t > nd:
+        _k().sm_window_attn_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                    block_tables.data_ptr(), block_tables.shape[1], sb.cu.data_ptr(),
+                                    sb.positions.data_ptr(), nd, sb.num_seqs, t, sb.max_q_len, h, g, d, dv, bs,
+                                    int(window), float(scale), f, _stream())
+    return out
