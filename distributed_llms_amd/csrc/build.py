@@ -41,8 +41,10 @@ FILE_FLAGS = {"attention.hip": ["-fno-honor-nans"]}
 
 def kernel_flags(src: str):
     """hipcc flags of one csrc/kernels source (without includes / output)."""
+    # packed-FP32 VALU forms (v_pk_*_f32) are kept out of every kernel: ordinary float code is
+    # compiled to the scalar forms
     common = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Wno-unused-result",
-              "-mcode-object-version=5"]
+              "-mcode-object-version=5", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
     if os.environ.get("DLLM_PART_TYPE"):        # split-K slab type (common.h); rebuild with force=True
         common.append(f"-DDLLM_PART_TYPE={int(os.environ['DLLM_PART_TYPE'])}")
     return common + FILE_FLAGS.get(os.path.basename(src), [])

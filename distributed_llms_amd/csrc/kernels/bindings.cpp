@@ -38,6 +38,17 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("paged_attention_decode", &dllm::paged_attention_decode);
   m.def("paged_attention_decode_rope", &dllm::paged_attention_decode_rope);
   m.def("paged_attention_prefill", &dllm::paged_attention_prefill);
+  m.def("sm_embed_f32", &dllm::sm_embed_f32);
+  m.def("sm_rms_norm", &dllm::sm_rms_norm);
+  m.def("sm_post_norm_add", &dllm::sm_post_norm_add);
+  m.def("sm_causal_conv", &dllm::sm_causal_conv);
+  m.def("sm_rglru_gates", &dllm::sm_rglru_gates);
+  m.def("sm_rglru_scan", &dllm::sm_rglru_scan);
+  m.def("sm_clipped_glu", &dllm::sm_clipped_glu);
+  m.def("sm_softcap", &dllm::sm_softcap);
+  m.def("sm_attn_prep", &dllm::sm_attn_prep);
+  m.def("sm_window_attn_decode", &dllm::sm_window_attn_decode);
+  m.def("sm_window_attn_prefill", &dllm::sm_window_attn_prefill);
   m.def("p2p_inbox_bytes", &dllm::p2p_inbox_bytes);
   m.def("p2p_standin", &dllm::p2p_standin);
   m.def("p2p_host_words", &dllm::p2p_host_words);

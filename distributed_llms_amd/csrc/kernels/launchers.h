@@ -67,6 +67,39 @@ void paged_attention_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uint
                              int hq, int hkv, int d, int block_size, int max_blocks, int max_q_len, float scale,
                              int version, uintptr_t positions, uintptr_t cos_sin, int q_stride, uintptr_t stream);
 
+// ---- layer-list models with per-sequence state (seqmix.hip, attention_window.hip); f32: activations
+// are float (else bf16)
+void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int width, int vocab, int f32,
+                  uintptr_t stream);
+void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, float eps, float offset, int f32,
+                 uintptr_t stream);
+void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
+                      int rows, int width, float eps, float mult, int f32, uintptr_t stream);
+void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,
+                    uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
+                    int tokens, int seqs, int C, int taps, int f32, int out_f32, uintptr_t stream);
+void sm_rglru_gates(uintptr_t a, uintptr_t g, uintptr_t u, uintptr_t ra_t, uintptr_t ra_b, uintptr_t ri_t,
+                    uintptr_t ri_b, uintptr_t lam, int tokens, int nb, int bw, float scale, int f32,
+                    uintptr_t stream);
+void sm_rglru_scan(uintptr_t out, uintptr_t a, uintptr_t g, uintptr_t y_raw, long y_stride, uintptr_t y_bias,
+                   uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t slots, int seqs, int C, int max_q_len,
+                   int f32, uintptr_t stream);
+void sm_clipped_glu(uintptr_t out, uintptr_t gu, uintptr_t bias, int tokens, int F, float limit, float alpha, int f32,
+                    uintptr_t stream);
+void sm_softcap(uintptr_t out, uintptr_t x, long n, float cap, int f32, uintptr_t stream);
+void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t state, uintptr_t q_norm,
+                  uintptr_t k_norm, uintptr_t freqs, int nrot, float mag, float eps, uintptr_t k_cache,
+                  uintptr_t v_cache, uintptr_t slot_mapping, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq,
+                  uintptr_t slots, int tokens, int seqs, int H, int G, int D, int Dv, int taps, int bs, int f32,
+                  uintptr_t stream);
+void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
+                           int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
+                           int Dv, int bs, int window, float scale, int f32, uintptr_t stream);
+void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
+                            int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
+                            int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, float scale,
+                            int f32, uintptr_t stream);
+
 long p2p_inbox_bytes(long chunk, int nslots);
 void p2p_standin(uintptr_t src, uintptr_t s_inbox, long s_bytes, uint64_t s_seq0, uintptr_t dst, uintptr_t r_inbox,
                  long r_bytes, uint64_t r_seq0, long chunk, int nslots, int channels, uintptr_t abort_word,

@@ -387,6 +387,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     if t > nd:
         _k().sm_window_attn_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                     block_tables.data_ptr(), block_tables.shape[1], sb.cu.data_ptr(),
-                                    sb.positions.data_ptr(), nd, sb.num_seqs, t, sb.max_q_len, h, g, d, dv, bs,
+                                    sb.positions.data_ptr(), sb.tok_seq.data_ptr(), nd, sb.num_seqs, t, sb.max_q_len,
+                                    h, g, d, dv, bs,
                                     int(window), float(scale), f, _stream())
     return out
