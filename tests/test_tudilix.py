@@ -1,0 +1,440 @@
+"""The layer-list hybrid model (sliding-window attention + RG-LRU layers) against the plain float64
+oracle of tests/oracle_tudilix.py: every mechanism alone, then the engine -- whole prompts,
+token-by-token decoding, prompt portions of several sizes, batches of unequal requests, blocks and
+state slots that are used again, window edges, long decoding, and greedy generation through the
+scheduler.  Each case runs on the CPU path in float32 and, marked gpu, on the HIP kernels in float32
+and bfloat16.
+"""
+import json
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import oracle_tudilix as O
+from distributed_llms_amd.config import EngineConfig, ModelConfig
+from distributed_llms_amd.engine.llm_engine import LLMEngine
+from distributed_llms_amd.engine.replay import TraceReplayer
+from distributed_llms_amd.engine.sequence import SamplingParams
+from distributed_llms_amd.models import make_stage
+from distributed_llms_amd.ops import seqmix as sm
+
+gpu = pytest.mark.gpu
+TARGETS = [pytest.param(("cpu", torch.float32), id="cpu-f32"),
+           pytest.param(("cuda", torch.float32), id="gpu-f32", marks=gpu),
+           pytest.param(("cuda", torch.bfloat16), id="gpu-bf16", marks=gpu)]
+
+
+def _rot(dims, scaling=True, base=10000.0):
+    r = {"base": base, "dims": dims}
+    if scaling:
+        r["scaling"] = {"factor": 6.0, "fast": 24.0, "original": 256, "slow": 2.0}
+    return r
+
+
+def cfg_a():
+    """Two attention layers of DIFFERENT shapes (one shares the first's K/V), grouped K/V heads,
+    value heads wider than key heads, rotation on part of the head, layers with and without a
+    feed-forward, RG-LRU layers with different taps and block counts."""
+    return {"architecture": "Tudilix", "vocab": 200, "width": 96, "residual_mult": 0.6, "logit_softcap": 12.0,
+            "norm": {"eps": 1e-6},
+            "layers": [
+                {"type": "attention", "mixer": {"conv": 3, "dim": 24, "vdim": 40, "heads": 4, "kv_heads": 2,
+                                                "mask": {"size": 37}, "scale": 0.3, "rot": _rot(12)},
+                 "mlp": {"kind": "dense", "ff": 160, "limit": 1.2}},
+                {"type": "rglru", "mixer": {"blocks": 3, "conv": 4, "width": 144}, "mlp": None},
+                {"type": "attention", "mixer": {"conv": 2, "dim": 24, "vdim": 40, "heads": 6, "kv_heads": 2, "kv_from": 0,
+                                                "mask": {"size": 9}, "scale": 0.2, "rot": _rot(24, scaling=False)},
+                 "mlp": None},
+                {"type": "rglru", "mixer": {"blocks": 2, "conv": 2, "width": 64},
+                 "mlp": {"kind": "dense", "ff": 72, "limit": 3.0}},
+            ]}
+
+
+def cfg_b():
+    """Degenerate sizes: one tap (a convolution that is a scale), one block, one K/V head per query
+    head, a window longer than any test prompt, no soft cap, residual_mult 1, odd widths."""
+    return {"architecture": "Tudilix", "vocab": 131, "width": 72, "residual_mult": 1.0, "logit_softcap": 0.0,
+            "norm": {"eps": 1e-5},
+            "layers": [
+                {"type": "rglru", "mixer": {"blocks": 1, "conv": 1, "width": 40},
+                 "mlp": {"kind": "dense", "ff": 56, "limit": 0.8}},
+                {"type": "attention", "mixer": {"conv": 1, "dim": 20, "vdim": 12, "heads": 3, "kv_heads": 3,
+                                                "mask": {"size": 4096}, "scale": 0.25, "rot": _rot(20)},
+                 "mlp": {"kind": "dense", "ff": 88, "limit": 5.0}},
+                {"type": "attention", "mixer": {"conv": 5, "dim": 16, "vdim": 16, "heads": 2, "kv_heads": 1,
+                                                "mask": {"size": 3}, "scale": 0.5, "rot": _rot(8, base=500.0)},
+                 "mlp": None},
+            ]}
+
+
+CONFIGS = {"a": cfg_a, "b": cfg_b}
+
+
+def _round(sd, dtype):
+    """Weights as the engine will hold them (rounded to bf16 for a bf16 run), for engine and oracle."""
+    return {k: torch.from_numpy(v).to(dtype).float() for k, v in sd.items()}
+
+
+def make_engine(cfg, sd, target, tmp_path, max_tokens=512, max_requests=4, block_size=32):
+    device, dtype = target
+    if device == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    mcfg = ModelConfig.from_hf_config(cfg)
+    stage = make_stage(mcfg, device=device, dtype=dtype).load_hf_state(sd)
+    ecfg = EngineConfig(model=str(tmp_path), shard_dir=str(tmp_path), device=device,
+                        dtype="float32" if dtype == torch.float32 else "bfloat16", max_batch=max_requests,
+                        max_seq_len=max_tokens + 1, kv_block_size=block_size,
+                        num_kv_blocks=-(-max_tokens // block_size) + max_requests + 1,
+                        max_prefill_tokens=max_tokens, use_graphs=False)
+    return LLMEngine(ecfg, stage)
+
+
+def rel_err(got, want):
+    """rms of the difference (mean over the vocabulary taken off) over the rms of the oracle's logits."""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = got - want
+    d = d - d.mean(-1, keepdims=True)
+    return float(np.sqrt((d ** 2).mean(-1)).max() / np.sqrt((want ** 2).mean()))
+
+
+def tol(target):
+    return 3e-5 if target[1] == torch.float32 else 3e-2
+
+
+def replay(engine, schedule, prompts):
+    """schedule: steps, each a list of (request name, token count); returns name -> logits [len, V]."""
+    rp = TraceReplayer(engine)
+    at = {n: 0 for n in prompts}
+    out = {n: [] for n in prompts}
+    for step in schedule:
+        entries, end = [], []
+        for n, c in step:
+            toks = prompts[n][at[n]:at[n] + c]
+            entries.append((n, toks, list(range(len(toks)))))
+            at[n] += c
+            if at[n] == len(prompts[n]):
+                end.append(n)
+        logits = rp.step(entries, end).cpu().numpy()
+        row = 0
+        for n, toks, _ in entries:
+            out[n].append(logits[row:row + len(toks)])
+            row += len(toks)
+    return {n: np.concatenate(v) for n, v in out.items() if v}
+
+
+def prompts_for(cfg, lens, seed=1):
+    rng = np.random.default_rng(seed)
+    return {f"r{i}": rng.integers(0, cfg["vocab"], n).tolist() for i, n in enumerate(lens)}
+
+
+# ------------------------------------------------------------------------------ mechanisms alone
+def _sb(chunks, device, slots=None):
+    """SeqBatch for chunks [(start position, length)]."""
+    cu = np.concatenate([[0], np.cumsum([n for _, n in chunks])]).astype(np.int32)
+    pos = np.concatenate([np.arange(s, s + n) for s, n in chunks]).astype(np.int32)
+    seq = np.concatenate([np.full(n, i) for i, (_, n) in enumerate(chunks)]).astype(np.int32)
+    slots = np.asarray(slots if slots is not None else range(1, len(chunks) + 1), dtype=np.int32)
+    t = lambda a: torch.from_numpy(a).to(device)
+    return sm.SeqBatch(t(cu), t(pos), t(seq), t(slots), len(chunks), int(cu[-1]), max(n for _, n in chunks))
+
+
+def _dev(target):
+    if target[0] == "cuda" and not torch.cuda.is_available():
+        pytest.skip("no GPU")
+    return target
+
+
+@pytest.mark.parametrize("target", TARGETS)
+def test_norms(target):
+    device, dtype = _dev(target)
+    rng = np.random.default_rng(0)
+    for width in (72, 200, 1030):
+        x = rng.standard_normal((5, width)).astype(np.float32) * 3
+        o = torch.from_numpy(rng.standard_normal((5, width)).astype(np.float32)).to(dtype)
+        w1, w2, b = (torch.from_numpy(0.2 * rng.standard_normal(width).astype(np.float32)).to(dtype) for _ in range(3))
+        y = sm.rms_norm_f32(torch.from_numpy(x).to(device), w1.to(device), 1e-5, dtype)
+        np.testing.assert_allclose(y.float().cpu().numpy(), O.rms(x.astype(np.float64), w1.float().numpy(), 1e-5, 1.0),
+                                   rtol=1e-5 if dtype == torch.float32 else 1e-2, atol=1e-5 if dtype == torch.float32 else 2e-2)
+        y = sm.rms_norm_f32(torch.from_numpy(x).to(device), w1.to(device), 1e-5, dtype, one_plus=False)
+        np.testing.assert_allclose(y.float().cpu().numpy(), O.rms(x.astype(np.float64), w1.float().numpy(), 1e-5, 0.0),
+                                   rtol=1e-5 if dtype == torch.float32 else 1e-2, atol=1e-5 if dtype == torch.float32 else 2e-2)
+        xr = torch.from_numpy(x.copy()).to(device)
+        xr, h = sm.post_norm_add(xr, o.to(device), w1.to(device), 1e-5, 0.5, bias=b.to(device), w_next=w2.to(device))
+        want_x = x + 0.5 * O.rms(o.float().numpy().astype(np.float64) + b.float().numpy(), w1.float().numpy(), 1e-5, 1.0)
+        np.testing.assert_allclose(xr.cpu().numpy(), want_x, rtol=1e-5, atol=1e-5)     # the residual stream is float32
+        np.testing.assert_allclose(h.float().cpu().numpy(), O.rms(want_x, w2.float().numpy(), 1e-5, 1.0),
+                                   rtol=1e-5 if dtype == torch.float32 else 1e-2, atol=1e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("taps", [1, 2, 4])
+def test_causal_conv_across_portions(target, taps):
+    """A sequence cut into portions (down to one token, shorter than the taps) equals the whole; a
+    second sequence in the same batch does not disturb it; slot content from a previous owner is not
+    read by a sequence that starts at 0."""
+    device, dtype = _dev(target)
+    rng = np.random.default_rng(taps)
+    c, n = 70, 23
+    u = torch.from_numpy(rng.standard_normal((n, c)).astype(np.float32)).to(dtype)
+    u2 = torch.from_numpy(rng.standard_normal((n, c)).astype(np.float32)).to(dtype)
+    w = torch.from_numpy(rng.standard_normal((c, taps)).astype(np.float32)).to(dtype)
+    b, ib = (torch.from_numpy(rng.standard_normal(c).astype(np.float32)).to(dtype) for _ in range(2))
+    want = O.causal_conv(u.float().numpy().astype(np.float64) + ib.float().numpy(), w.float().numpy(), b.float().numpy())
+    state = torch.full((4, taps - 1, c), 7.0, dtype=dtype, device=device)      # garbage from a previous owner
+    got, at, at2 = [], 0, 0
+    for k in (1, 1, 2, 1, 5, 3, 10):
+        pieces = [u[at:at + k]]
+        chunks = [(at, k)]
+        if at2 < n:                               # the other sequence advances by other amounts
+            k2 = min(n - at2, k + 2)
+            pieces.append(u2[at2:at2 + k2])
+            chunks.append((at2, k2))
+            at2 += k2
+        y = sm.causal_conv(torch.cat(pieces).to(device), w.to(device), b.to(device), state, _sb(chunks, device, [2, 1][:len(chunks)]),
+                           in_bias=ib.to(device))
+        got.append(y[:k].cpu().numpy())
+        at += k
+    np.testing.assert_allclose(np.concatenate(got), want, rtol=1e-5, atol=1e-5)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+def test_rglru_long_memory_across_portions(target):
+    """Slow decays (lam very negative): the first tokens still weigh on the state hundreds of tokens
+    later, so a state that is lost or reset between portions shows at the end."""
+    device, dtype = _dev(target)
+    rng = np.random.default_rng(5)
+    nb, bw, n = 3, 20, 300
+    c = nb * bw
+    f = lambda *s: rng.standard_normal(s).astype(np.float32)
+    u, yraw = f(n, c), f(n, c)
+    ra, ri = f(nb, bw, bw) / math.sqrt(bw), f(nb, bw, bw) / math.sqrt(bw)
+    rab, rib, yb = 0.3 * f(nb, bw), 0.3 * f(nb, bw), 0.2 * f(c)
+    lam = rng.uniform(-9.0, -5.0, c).astype(np.float32)
+    T = lambda a: torch.from_numpy(a).to(dtype)
+    ra, ri, rab, rib, yb, lam, yraw = (T(a) for a in (ra, ri, rab, rib, yb, lam, yraw))
+    # oracle
+    a64 = lambda t: t.float().numpy().astype(np.float64)
+    r = np.zeros((n, c)); ig = np.zeros((n, c))
+    for b in range(nb):
+        ub = u[:, b * bw:(b + 1) * bw].astype(np.float64)
+        r[:, b * bw:(b + 1) * bw] = O.sigmoid(ub @ a64(ra)[b].T + a64(rab)[b])
+        ig[:, b * bw:(b + 1) * bw] = O.sigmoid(ub @ a64(ri)[b].T + a64(rib)[b])
+    a = np.exp(-8.0 * r * O.softplus(a64(lam)))
+    s = np.zeros(c); want = np.zeros((n, c))
+    for i in range(n):
+        s = a[i] * s + np.sqrt(1 - a[i] ** 2) * ig[i] * u[i]
+        want[i] = s * O.gelu_tanh(a64(yraw)[i] + a64(yb))
+    assert abs(a.min()) > 0.9          # decays are slow: position 0 matters at the end
+    state = torch.full((3, c), 5.0, dtype=torch.float32, device=device)
+    got, at = [], 0
+    for k in (2, 1, 64, 1, 1, 100, 3, 128):
+        sb = _sb([(at, k)], device, [2])
+        o = sm.rglru(torch.from_numpy(u[at:at + k]).to(device), yraw[at:at + k].to(device), yb.to(device),
+                     ra.transpose(1, 2).contiguous().to(device), rab.to(device), ri.transpose(1, 2).contiguous().to(device),
+                     rib.to(device), lam.to(device), state, sb, dtype)
+        got.append(o.float().cpu().numpy())
+        at += k
+    assert at == n
+    np.testing.assert_allclose(np.concatenate(got), want, rtol=2e-4 if dtype == torch.float32 else 2e-2,
+                               atol=2e-5 if dtype == torch.float32 else 2e-2)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+def test_clipped_glu_and_softcap(target):
+    device, dtype = _dev(target)
+    rng = np.random.default_rng(2)
+    f = 37
+    gu = torch.from_numpy(3 * rng.standard_normal((9, 2 * f)).astype(np.float32)).to(dtype)
+    b = torch.from_numpy(rng.standard_normal(2 * f).astype(np.float32)).to(dtype)
+    x = gu.float().numpy().astype(np.float64) + b.float().numpy()
+    g, u = np.minimum(x[:, :f], 1.5), np.clip(x[:, f:], -1.5, 1.5)
+    want = g * O.sigmoid(1.702 * g) * (u + 1)
+    got = sm.clipped_glu(gu.to(device), b.to(device), 1.5).float().cpu().numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-5 if dtype == torch.float32 else 1e-2, atol=1e-5 if dtype == torch.float32 else 2e-2)
+    lg = torch.from_numpy(30 * rng.standard_normal((4, 50)).astype(np.float32)).to(dtype)
+    got = sm.softcap_f32(lg.to(device), 11.0).cpu().numpy()
+    np.testing.assert_allclose(got, 11.0 * np.tanh(lg.float().numpy().astype(np.float64) / 11.0), rtol=1e-5, atol=1e-5)
+    assert sm.softcap_f32(lg.to(device), 0.0).dtype == torch.float32
+
+
+def test_yarn_frequencies():
+    for rot in (_rot(12), _rot(24, scaling=False), _rot(8, base=500.0)):
+        f, mag = sm.yarn_frequencies(rot["dims"], rot["base"], rot.get("scaling"))
+        cos, sin = O.rotary_tables(rot, 50)
+        ang = np.arange(50)[:, None] * f.numpy().astype(np.float64)[None]
+        np.testing.assert_allclose(np.cos(ang) * mag, cos, atol=2e-5)
+        np.testing.assert_allclose(np.sin(ang) * mag, sin, atol=2e-5)
+
+
+def _paged(k, v, bs, device, dtype, num_blocks, table):
+    """Scatter per-position k [n, G, D] / v [n, G, Dv] into paged caches following ``table``."""
+    n, g, d = k.shape
+    kc = torch.zeros(num_blocks, g, bs, d, dtype=dtype)
+    vc = torch.zeros(num_blocks, g, bs, v.shape[2], dtype=dtype)
+    for j in range(n):
+        kc[table[j // bs], :, j % bs] = k[j]
+        vc[table[j // bs], :, j % bs] = v[j]
+    return kc.to(device), vc.to(device)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("window", [1, 7, 32, 33, 300])
+def test_window_edges_with_a_dominant_key(target, window):
+    """One key gets a score far above the rest.  Placed just inside the window (p - window + 1) it owns
+    the output; just outside (p - window) it must not be seen at all -- in a prompt portion and for a
+    decoded token, with the edge inside a block and on a block border, blocks scattered in the pool."""
+    device, dtype = _dev(target)
+    rng = np.random.default_rng(window)
+    n, h, g, d, dv, bs = 140, 4, 2, 24, 40, 16
+    q = rng.standard_normal((n, h, d)).astype(np.float32)
+    k = rng.standard_normal((n, g, d)).astype(np.float32)
+    v = rng.standard_normal((n, g, dv)).astype(np.float32)
+    table = list(rng.permutation(np.arange(1, 40))[:-(-n // bs)])
+    T = lambda a: torch.from_numpy(a).to(dtype)
+    for p in (n - 1, 97, 64, 63):
+        for inside in (True, False):
+            j = p - window + (1 if inside else 0)
+            if j < 0:
+                continue
+            k2 = k.copy()
+            k2[j] = 0.0
+            k2[j, :, 0] = 60.0                       # with q[p, :, 0] = 1: a score 60 * scale above the rest
+            q2 = q.copy()
+            q2[p, :, 0] = 1.0
+            qq, kk, vv = T(q2), T(k2), T(v)
+            want = O.window_attention(qq.float().numpy().astype(np.float64), kk.float().numpy().astype(np.float64),
+                                      vv.float().numpy().astype(np.float64), window, 0.5)
+            kc, vc = _paged(kk, vv, bs, device, dtype, 40, table)
+            bt = torch.tensor([table], dtype=torch.int32, device=device)
+            t = 1e-5 if dtype == torch.float32 else 2e-2
+            # the last 12 positions up to p as a prompt portion
+            lo = max(0, p - 11)
+            sb = _sb([(lo, p + 1 - lo)], device)
+            o = sm.window_attention(qq[lo:p + 1].contiguous().to(device), kc, vc, bt, sb, window, 0.5, num_decode=0)
+            np.testing.assert_allclose(o.float().cpu().numpy(), want[lo:p + 1], rtol=t, atol=t)
+            # position p as a decoded token
+            sb = _sb([(p, 1)], device)
+            o = sm.window_attention(qq[p:p + 1].contiguous().to(device), kc, vc, bt, sb, window, 0.5)
+            np.testing.assert_allclose(o.float().cpu().numpy(), want[p:p + 1], rtol=t, atol=t)
+            if inside and window > 1:
+                np.testing.assert_allclose(want[p, 0], vv[j, 0].float().numpy(), atol=1e-3)   # the test bites
+
+
+# ------------------------------------------------------------------------------ the engine
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_whole_prompts_and_layers(target, name, tmp_path):
+    cfg = CONFIGS[name]()
+    sd = _round(O.make_weights(cfg, seed=3), target[1])
+    eng = make_engine(cfg, sd, target, tmp_path)
+    prompts = prompts_for(cfg, [1, 2, 45, 130])
+    eng.stage.taps = []
+    got = replay(eng, [[(n, len(p))] for n, p in prompts.items()], prompts)
+    taps = eng.stage.taps
+    eng.stage.taps = None
+    nl = len(cfg["layers"])
+    for i, (n, p) in enumerate(prompts.items()):
+        want, layers = O.forward(cfg, sd, p)
+        assert rel_err(got[n], want) < tol(target), n
+        if target[1] == torch.float32:            # the residual stream after every layer
+            mine = torch.stack(taps[i * nl:(i + 1) * nl]).cpu().numpy()
+            np.testing.assert_allclose(mine, layers, rtol=2e-4, atol=2e-4)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("name", ["a", "b"])
+def test_decode_and_portions_match_the_whole(target, name, tmp_path):
+    """Token-by-token decoding after a prompt (long enough that the windows pass over decoded tokens),
+    and portions of changing sizes down to two tokens and one, cut inside blocks and windows."""
+    cfg = CONFIGS[name]()
+    sd = _round(O.make_weights(cfg, seed=4), target[1])
+    eng = make_engine(cfg, sd, target, tmp_path)
+    p = prompts_for(cfg, [150], seed=7)
+    want, _ = O.forward(cfg, sd, p["r0"])
+    got = replay(eng, [[("r0", 60)]] + [[("r0", 1)]] * 90, p)
+    assert rel_err(got["r0"], want) < tol(target)
+    sizes = [2, 3, 1, 31, 2, 33, 5, 64, 2, 7]
+    assert sum(sizes) == 150
+    got = replay(eng, [[("r0", s)] for s in sizes], p)
+    assert rel_err(got["r0"], want) < tol(target)
+    got = replay(eng, [[("r0", 1)]] * 40, {"r0": p["r0"][:40]})        # from the very first token on
+    assert rel_err(got["r0"], want[:40]) < tol(target)
+
+
+@pytest.mark.parametrize("target", TARGETS)
+def test_mixed_batches_and_reused_blocks_and_slots(target, tmp_path):
+    """Up to four unequal requests per step, portions beside single tokens; finished requests give
+    their blocks and state slot to new ones (a pool sized for the live tokens only).  Every request
+    matches its own whole-sequence oracle, i.e. the batch and the pool do not show."""
+    cfg = cfg_a()
+    sd = _round(O.make_weights(cfg, seed=5), target[1])
+    eng = make_engine(cfg, sd, target, tmp_path, max_tokens=288, max_requests=4)
+    lens = [70, 9, 33, 64, 20, 50, 3]
+    prompts = prompts_for(cfg, lens, seed=9)
+    names = list(prompts)
+    at = {n: 0 for n in names}
+    waiting, live, schedule = list(names), [], []
+    rng = np.random.default_rng(0)
+    while waiting or live:
+        while waiting and len(live) < 4:
+            live.append(waiting.pop(0))
+        step = []
+        for n in list(live):
+            left = len(prompts[n]) - at[n]
+            c = min(left, int(rng.choice([1, 1, 2, 3, 17, 32])))
+            if rng.random() < 0.15 and len(live) > 1:
+                continue                                # left out of this step, goes on later
+            step.append((n, c))
+            at[n] += c
+            if at[n] == len(prompts[n]):
+                live.remove(n)
+        if step:
+            schedule.append(step)
+    got = replay(eng, schedule, prompts)
+    assert eng.bm.num_free() == eng.bm.num_blocks - 1 and eng.bm.num_free_state_slots() == 4   # all given back
+    for n in names:
+        want, _ = O.forward(cfg, sd, prompts[n])
+        assert rel_err(got[n], want) < tol(target), n
+
+
+@pytest.mark.parametrize("target", TARGETS)
+def test_greedy_generation_through_the_scheduler(target, tmp_path):
+    """LLMEngine.generate (scheduler, continuous batching, sampler) on three prompts at once: every
+    generated token is the argmax of the oracle's logits for the sequence so far (where the oracle's
+    top two are not within rounding of each other)."""
+    cfg = cfg_a()
+    sd = _round(O.make_weights(cfg, seed=6), target[1])
+    eng = make_engine(cfg, sd, target, tmp_path)
+    prompts = list(prompts_for(cfg, [5, 40, 17], seed=11).values())
+    outs = eng.generate(prompts, SamplingParams(max_new_tokens=24, ignore_eos=True))
+    margin = 1e-3 if target[1] == torch.float32 else 0.3
+    for p, o in zip(prompts, outs):
+        assert len(o) == 24
+        logits, _ = O.forward(cfg, sd, p + o)
+        for i, tok in enumerate(o):
+            row = logits[len(p) + i - 1]
+            top = np.sort(row)[-2:]
+            if top[1] - top[0] > margin:
+                assert tok == int(row.argmax()), (i, tok, int(row.argmax()))
+    assert eng.bm.num_free_state_slots() == eng.bm.num_state_slots - 1      # only the scratch slot is held
+
+
+def test_config_round_trip_and_registry(tmp_path):
+    from distributed_llms_amd.config import get_model_config
+    from distributed_llms_amd.models.hybrid import HybridStage, model_shapes
+    cfg = cfg_a()
+    (tmp_path / "config.json").write_text(json.dumps(cfg))
+    m = get_model_config(str(tmp_path))
+    assert m.arch == "tudilix" and m.num_layers == 4 and m.hidden_size == 96 and m.needs_state_slots
+    assert ModelConfig.from_hf_config(m.to_hf_config()).layers == m.layers
+    assert isinstance(make_stage(m), HybridStage)
+    sd = O.make_weights(cfg)
+    assert {k: tuple(v.shape) for k, v in sd.items()} == model_shapes(m)
+    with pytest.raises(ValueError):
+        bad = cfg_a()
+        bad["layers"][2]["mixer"]["kv_from"] = 1      # not an attention layer
+        make_stage(ModelConfig.from_hf_config(bad))
+    assert get_model_config("tiny-tudilix").arch == "tudilix"
