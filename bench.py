@@ -84,6 +84,10 @@ def parse(argv=None):
     ap.add_argument("--trace", default=None, metavar="DIR",
                     help="record a roctx/host/GPU timeline of the timed steps: DIR/trace_rank<r>.json "
                          "(Chrome format) and per-stage device busy %% in the JSON line")
+    ap.add_argument("--hybrid", default=None, metavar="SIZE[,SIZE]",
+                    help="instead of the headline workload: prefill and decode tokens/s of the layer-list hybrid "
+                         "model (Tudilix) beside a Llama-architecture model of equal size (sizes: 2b, 9b, small), "
+                         "--batch prompts of --prompt-len tokens then --gen-len decode steps; one JSON line per size")
     return ap.parse_args(argv)
 
 
@@ -353,6 +357,12 @@ def main(argv=None):
         import faulthandler
         faulthandler.dump_traceback_later(args.hang_dump, repeat=True)
     world = int(os.environ.get("WORLD_SIZE", "1"))
+    if args.hybrid:
+        from distributed_llms_amd.engine import hybrid_bench
+        for size in args.hybrid.split(","):
+            print(json.dumps(hybrid_bench.run(size, args.batch, args.prompt_len, args.gen_len, max(1, args.steps - 1))),
+                  flush=True)
+        return None
     if args.rate > 0:
         if world > 1 or args.gpus > 1:
             raise SystemExit("--rate (open-loop latency mode) runs on one GPU")

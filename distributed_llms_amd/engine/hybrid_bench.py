@@ -1,0 +1,96 @@
+"""Prefill and decode throughput of the layer-list hybrid model beside a Llama-architecture model of
+equal size (``bench.py --hybrid``): same width, layer count, feed-forward size, head size and K/V
+heads, random weights, one GPU.  Every step goes through the engine's StageRunner (the trace
+replayer builds the batches): one step with ``batch`` prompts of ``prompt_len`` tokens (prefill),
+then ``gen_len`` steps of one token per sequence (decode)."""
+from __future__ import annotations
+
+import json
+import time
+
+import numpy as np
+import torch
+
+from ..config import EngineConfig, ModelConfig
+from ..models import make_stage
+from .llm_engine import LLMEngine
+from .replay import TraceReplayer
+
+# name -> (width, layers, ff, heads, kv_heads, head size, rglru blocks, window)
+SIZES = {
+    "2b": (2560, 6, 7680, 20, 4, 128, 10, 2048),
+    "9b": (4096, 6, 12288, 32, 8, 128, 16, 2048),
+    "small": (1024, 6, 3072, 8, 2, 128, 4, 512),
+}
+
+
+def hybrid_config(size: str, vocab: int = 32000) -> ModelConfig:
+    w, nl, ff, h, g, d, nb, win = SIZES[size]
+    rot = {"base": 10000.0, "dims": d // 2, "scaling": {"factor": 4.0, "fast": 32.0, "original": 4096, "slow": 1.0}}
+    layers = []
+    for i in range(nl):
+        mlp = {"kind": "dense", "ff": ff, "limit": 7.0}
+        if i % 3 == 2:
+            layers.append({"type": "attention", "mlp": mlp, "mixer": {
+                "conv": 4, "dim": d, "vdim": d, "heads": h, "kv_heads": g, "mask": {"size": win},
+                "scale": d ** -0.5, "rot": rot}})
+        else:
+            layers.append({"type": "rglru", "mlp": mlp, "mixer": {"blocks": nb, "conv": 4, "width": w}})
+    return ModelConfig.from_hf_config({"architecture": "Tudilix", "vocab": vocab, "width": w, "residual_mult": 1.0,
+                                       "logit_softcap": 30.0, "norm": {"eps": 1e-6}, "layers": layers},
+                                      name=f"tudilix-{size}")
+
+
+def llama_config(size: str, vocab: int = 32000) -> ModelConfig:
+    w, nl, ff, h, g, d, _nb, _win = SIZES[size]
+    return ModelConfig(name=f"llama-{size}", arch="llama", vocab_size=vocab, hidden_size=w, intermediate_size=ff,
+                       num_layers=nl, num_heads=h, num_kv_heads=g, head_dim=d, max_position=8192)
+
+
+def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps: int, tmp: str, graphs: bool):
+    import os
+    os.makedirs(tmp, exist_ok=True)
+    with open(os.path.join(tmp, "config.json"), "w") as f:
+        json.dump(mcfg.to_hf_config(), f)
+    stage = make_stage(mcfg, device="cuda", dtype=torch.bfloat16).init_synthetic(0)
+    total = batch * (prompt_len + gen_len + 32)
+    ecfg = EngineConfig(model=tmp, shard_dir=tmp, device="cuda", dtype="bfloat16", max_batch=batch,
+                        max_seq_len=prompt_len + gen_len + 8, kv_block_size=32,
+                        num_kv_blocks=-(-total // 32) + batch + 2, max_prefill_tokens=batch * prompt_len,
+                        use_graphs=graphs, graph_batch_sizes=(batch,))
+    eng = LLMEngine(ecfg, stage)
+    rp = TraceReplayer(eng)
+    rng = np.random.default_rng(0)
+    pre, dec = [], []
+    for r in range(reps + 1):
+        names = [f"q{r}_{i}" for i in range(batch)]
+        toks = rng.integers(10, mcfg.vocab_size - 1, size=(batch, prompt_len + gen_len)).tolist()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        rp.step([(n, toks[i][:prompt_len], [prompt_len - 1]) for i, n in enumerate(names)])
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        for k in range(gen_len):
+            rp.step([(n, [toks[i][prompt_len + k]], [0]) for i, n in enumerate(names)],
+                    end=names if k == gen_len - 1 else ())
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if r:                   # the first round warms up (allocations, graph capture)
+            pre.append(t1 - t0)
+            dec.append(t2 - t1)
+    del eng, rp, stage
+    torch.cuda.empty_cache()
+    return batch * prompt_len / min(pre), batch * gen_len / min(dec)
+
+
+def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int = 32, reps: int = 2,
+        tmp: str = "/tmp/dllm_hybrid_bench") -> dict:
+    out = {"size": size, "batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
+           "data": "synthetic (random-init weights, random token ids)"}
+    for key, cfg, graphs in (("tudilix", hybrid_config(size), False), ("llama", llama_config(size), True)):
+        p, d = _measure(cfg, batch, prompt_len, gen_len, reps, f"{tmp}/{key}", graphs)
+        out[key] = {"prefill_tok_s": round(p, 1), "decode_tok_s": round(d, 1),
+                    "params_m": round(cfg.param_count() / 1e6, 1)}
+    out["prefill_ratio"] = round(out["tudilix"]["prefill_tok_s"] / out["llama"]["prefill_tok_s"], 3)
+    out["decode_ratio"] = round(out["tudilix"]["decode_tok_s"] / out["llama"]["decode_tok_s"], 3)
+    return out
