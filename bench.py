@@ -88,6 +88,7 @@ def parse(argv=None):
                     help="instead of the headline workload: prefill and decode tokens/s of the layer-list hybrid "
                          "model (Tudilix) beside a Llama-architecture model of equal size (sizes: 2b, 9b, small), "
                          "--batch prompts of --prompt-len tokens then --gen-len decode steps; one JSON line per size")
+    ap.add_argument("--hybrid-models", default="tudilix,llama", help="--hybrid: which of the two models to run")
     return ap.parse_args(argv)
 
 
@@ -360,7 +361,8 @@ def main(argv=None):
     if args.hybrid:
         from distributed_llms_amd.engine import hybrid_bench
         for size in args.hybrid.split(","):
-            print(json.dumps(hybrid_bench.run(size, args.batch, args.prompt_len, args.gen_len, max(1, args.steps - 1))),
+            print(json.dumps(hybrid_bench.run(size, args.batch, args.prompt_len, args.gen_len, max(1, args.steps - 1),
+                                              models=tuple(args.hybrid_models.split(",")))),
                   flush=True)
         return None
     if args.rate > 0:

@@ -1,5 +1,6 @@
 // Sliding-window attention over a paged K/V cache whose key and value head sizes differ
-// (ops/seqmix.py window_attention): caches k [NB, G, BS, D], v [NB, G, BS, Dv] (one row per key),
+// (ops/seqmix.py window_attention): caches k [NB, G, BS, D] (one row per key), v [NB, G, Dv, BS]
+// (transposed inside a block: 8 keys of one value channel are one 16-byte load),
 // query head h reads K/V head h / (H / G), a query at position p sees the keys j of its sequence with
 // 0 <= p - j < window.  Scores, softmax weights and the weighted sum are float32; T is the storage
 // type (bf16 or float).  Head sizes, window and block size are runtime values.
@@ -7,7 +8,14 @@
 //   window_attn_row_kernel   one workgroup per (query token, head): keys in tiles of 256, one key per
 //                            thread for q.k, an online softmax across tiles, then P.V with the
 //                            threads laid out (value channel, key subgroup).  Decode rows, and prompt
-//                            chunks too short to fill a query tile.
+//                            chunks in float32.
+//   window_attn_tile_kernel  bf16 prompt chunks on MFMA (v_mfma_f32_16x16x32_bf16): one workgroup per
+//                            (64-query tile of a chunk, head), 4 waves x 16 queries, keys in tiles of 32
+//                            staged through LDS (K rows permuted so that the S^T = K Q^T accumulator
+//                            hands each lane 8 consecutive keys, V transposed so that P.V reads 8 keys
+//                            of one value channel in one 16-byte load).  The softmax weights stay
+//                            float32: P is fed to the matrix cores as a bf16 pair (high part + the
+//                            rounding remainder), two MFMAs per tile, so P.V carries 16 significand bits.
 #include <math.h>
 
 #include "common.h"
@@ -98,7 +106,7 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
     if (j <= pos) {
       const int blk = bt[j / bs];
       const int row = (blk * G + g) * bs + (j % bs);
-      rows[tid] = row;
+      rows[tid] = row;                                      // K row; V element (e) at ((row / bs) * Dv + e) * bs + row % bs
       s = dot_row<T>(qs, kc + (size_t)row * D, D) * scale;
     }
     const float m_new = fmaxf(m, block_max(s, red));
@@ -114,7 +122,10 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
       const int e = e0 + i * ew;
       if (sub < nsub && e < Dv) {
         float a = acc[i] * corr;
-        for (int k = sub; k < nk; k += nsub) a = fmaf(p[k], wld(vc + (size_t)rows[k] * Dv + e), a);
+        for (int k = sub; k < nk; k += nsub) {
+          const int row = rows[k], hb = row / bs;
+          a = fmaf(p[k], wld(vc + ((size_t)hb * Dv + e) * bs + (row - hb * bs)), a);
+        }
         acc[i] = a;
       }
     }
@@ -161,11 +172,313 @@ static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
+
+// --------------------------------------------------------------------------- MFMA prompt kernel (bf16)
+constexpr int kTQ = 64;          // queries per workgroup (16 per wave)
+constexpr int kTK = 32;          // keys per tile
+constexpr int kPad = 8;          // bf16 elements of row padding in LDS (16 bytes: rows start on different banks)
+
+// NQK: 32-wide K-dim steps of q.k (D <= 32 NQK); NDV: 16-wide tiles of value channels (Dv <= 16 NDV)
+template <int NQK, int NDV>
+__global__ void __launch_bounds__(256) window_attn_tile_kernel(
+    bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+    const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int H, int G, int D, int Dv,
+    int bs, int window, float scale) {
+  constexpr int DP = 32 * NQK, KROW = DP + kPad, VROW = kTK + kPad;
+  __shared__ __attribute__((aligned(16))) bf16 ks[kTK * KROW];          // K tile, key j at row krow32(j)
+  __shared__ __attribute__((aligned(16))) bf16 vs[16 * NDV * VROW];     // V^T tile [channel][key]
+  const int b = seq0 + blockIdx.y, h = blockIdx.z;
+  const int lo_t = cu[b], n = cu[b + 1] - lo_t;
+  const int q0 = blockIdx.x * kTQ;                                     // first local query of the tile
+  if (q0 >= n) return;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, grp = lane >> 4;
+  const int g = h / (H / G);
+  const int start = positions[lo_t];                                   // position of the chunk's first token
+  const int32_t* bt = block_tables + (size_t)b * max_blocks;
+  // this lane's query (MFMA column): local index, position, validity
+  const int ql = q0 + wave * 16 + col;
+  const bool qok = ql < n;
+  const int qpos = start + min(ql, n - 1);
+  // Q fragments: B operand, lane (col, grp) holds q[query col][32 s + 8 grp .. + 7]
+  bf16x8 qf[NQK];
+  {
+    const bf16* qrow = q + ((size_t)(lo_t + min(ql, n - 1)) * H + h) * D;
+#pragma unroll
+    for (int s2 = 0; s2 < NQK; ++s2) {
+      const int d0 = 32 * s2 + 8 * grp;
+      bf16x8 v;
+      if (d0 + 8 <= D) v = *reinterpret_cast<const bf16x8*>(qrow + d0);
+      else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = d0 + j < D ? qrow[d0 + j] : (bf16)0.f;
+      }
+      qf[s2] = v;
+    }
+  }
+  // zero the K padding columns once (d in [D, DP)): the loads below never write them
+  for (int i = tid; i < kTK * KROW; i += 256) ks[i] = (bf16)0.f;
+  for (int i = tid; i < 16 * NDV * VROW; i += 256) vs[i] = (bf16)0.f;
+  f32x4 acc[NDV];
+#pragma unroll
+  for (int i = 0; i < NDV; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  const int last_pos = start + min(q0 + kTQ, n) - 1;                   // newest key any query of the tile sees
+  const int first_pos = max(0, start + q0 - window + 1);               // oldest
+  // this wave's queries see keys in [wlo, whi]
+  const int whi = start + min(q0 + wave * 16 + 15, n - 1), wlo = max(0, start + q0 + wave * 16 - window + 1);
+  const int d8 = D >> 3;
+  __syncthreads();
+  for (int k0 = first_pos & ~(kTK - 1); k0 <= last_pos; k0 += kTK) {
+    // ---- stage the tile: K rows (16-byte pieces), V transposed (element-wise)
+    for (int i = tid; i < kTK * d8; i += 256) {
+      const int j = i / d8, c = i - j * d8;
+      const int kp = min(k0 + j, last_pos);
+      const size_t row = ((size_t)bt[kp / bs] * G + g) * bs + (kp % bs);
+      *reinterpret_cast<bf16x8*>(ks + krow32(j) * KROW + 8 * c) =
+          *reinterpret_cast<const bf16x8*>(k_cache + row * D + 8 * c);
+    }
+    for (int i = tid; i < Dv * (kTK / 8); i += 256) {
+      const int ch = i / (kTK / 8), c = i - ch * (kTK / 8);
+      const int kp = min(k0 + 8 * c, last_pos & ~7);       // 8 keys of one block (bs % 8 == 0)
+      const size_t at = (((size_t)bt[kp / bs] * G + g) * Dv + ch) * bs + (kp % bs);
+      *reinterpret_cast<bf16x8*>(vs + ch * VROW + 8 * c) = *reinterpret_cast<const bf16x8*>(v_cache + at);
+    }
+    __syncthreads();
+    if (k0 <= whi && k0 + kTK - 1 >= wlo) {
+      // ---- S^T = K Q^T: lane (col, grp) gets keys k0 + 8 grp + (0..7) of query col
+      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int s2 = 0; s2 < NQK; ++s2) {
+        const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + col * KROW + 32 * s2 + 8 * grp);
+        const bf16x8 kb = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KROW + 32 * s2 + 8 * grp);
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[s2], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qf[s2], s1, 0, 0, 0);
+      }
+      float p[8];
+      float cm = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const int kp = k0 + 8 * grp + i;
+        const float sv = (i < 4 ? s0[i] : s1[i - 4]) * scale;
+        const bool ok = qok && kp <= qpos && qpos - kp < window;
+        p[i] = ok ? sv : -INFINITY;
+        cm = fmaxf(cm, p[i]);
+      }
+      cm = rows_max(cm);
+      const float m_new = fmaxf(m, cm);
+      const float m_use = m_new == -INFINITY ? 0.f : m_new;
+      const float alpha = m == -INFINITY ? 0.f : expf(m - m_new);
+      float ps = 0.f;
+      bf16x8 ph, pl;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float e = expf(p[i] - m_use);
+        ps += e;
+        ph[i] = (bf16)e;
+        pl[i] = (bf16)(e - (float)ph[i]);
+      }
+      l = l * alpha + rows_sum(ps);
+      m = m_new;
+#pragma unroll
+      for (int dt = 0; dt < NDV; ++dt) {
+        if (16 * dt < Dv) {
+          // A operand: V^T[channel 16 dt + col][keys 8 grp .. + 7]
+          const bf16x8 va = *reinterpret_cast<const bf16x8*>(vs + (16 * dt + col) * VROW + 8 * grp);
+          f32x4 a = acc[dt] * alpha;
+          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, ph, a, 0, 0, 0);
+          acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl, a, 0, 0, 0);
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // O^T accumulator: lane (col, grp) holds channels 16 dt + 4 grp + (0..3) of query col
+  if (!qok) return;
+  const float inv = 1.0f / l;
+  bf16* orow = out + ((size_t)(lo_t + ql) * H + h) * Dv;
+#pragma unroll
+  for (int dt = 0; dt < NDV; ++dt) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int e = 16 * dt + 4 * grp + i;
+      if (e < Dv) orow[e] = (bf16)(acc[dt][i] * inv);
+    }
+  }
+}
+
+template <int NQK, int NDV>
+static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
+                        int max_blocks, uintptr_t cu, uintptr_t positions, int seq0, int nseq, int max_q_len, int H,
+                        int G, int D, int Dv, int bs, int window, float scale, uintptr_t stream) {
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV>), dim3((max_q_len + kTQ - 1) / kTQ, nseq, H),
+                     dim3(256), 0, (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
+                     (const bf16*)v_cache, (const int32_t*)block_tables, max_blocks, (const int32_t*)cu,
+                     (const int32_t*)positions, seq0, H, G, D, Dv, bs, window, scale);
+  DLLM_HIP_CHECK(hipGetLastError());
+}
+
+
+// --------------------------------------------------------------------------- MFMA decode kernel (bf16)
+// One workgroup per (one-token sequence, K/V head): the 16 MFMA columns are the query heads of the
+// group, so the keys and values of a K/V head are read once for all of them.  The wave's key tiles
+// (32 keys, tile index mod kDW = wave) go from global memory straight into MFMA fragments: K rows as
+// the A operand of S^T = K Q^T (row r of a 16-key half holds the key that makes the accumulator hand
+// each lane 8 consecutive keys), V^T pieces (8 keys of one channel, 16 bytes) as the A operand of
+// O^T = V^T P^T.  Each wave keeps an online softmax; the waves' partial results meet in LDS.
+constexpr int kDW = 4;
+
+template <int NQK, int NDV>
+__global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
+    bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
+    const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int H, int G, int D, int Dv, int bs,
+    int window, float scale) {
+  constexpr int DVP = 16 * NDV;
+  __shared__ float so[kDW][16][DVP + 1];
+  __shared__ float sml[kDW][2][16];
+  const int t = blockIdx.x, g = blockIdx.y;
+  const int R = H / G;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, grp = lane >> 4;
+  const int pos = positions[t], b = tok_seq[t];
+  const int lo = max(0, pos - window + 1);
+  const int32_t* bt = block_tables + (size_t)b * max_blocks;
+  bf16x8 qf[NQK];
+  {
+    const bf16* qrow = q + ((size_t)t * H + g * R + min(col, R - 1)) * D;
+#pragma unroll
+    for (int s2 = 0; s2 < NQK; ++s2) {
+      const int d0 = 32 * s2 + 8 * grp;
+      bf16x8 v;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
+      if (d0 + 8 <= D && col < R) v = *reinterpret_cast<const bf16x8*>(qrow + d0);
+      qf[s2] = v;
+    }
+  }
+  f32x4 acc[NDV];
+#pragma unroll
+  for (int i = 0; i < NDV; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, l = 0.f;
+  // keys of this lane's A rows inside a tile: first half row col -> key 8 (col / 4) + col % 4, second half + 4
+  const int jr = 8 * (col >> 2) + (col & 3);
+  for (int k0 = (lo & ~31) + 32 * wave; k0 <= pos; k0 += 32 * kDW) {
+    const int j1 = min(k0 + jr, pos), j2 = min(k0 + jr + 4, pos);
+    const bf16* r1 = k_cache + (((size_t)bt[j1 / bs] * G + g) * bs + j1 % bs) * D;
+    const bf16* r2 = k_cache + (((size_t)bt[j2 / bs] * G + g) * bs + j2 % bs) * D;
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s2 = 0; s2 < NQK; ++s2) {
+      const int d0 = 32 * s2 + 8 * grp;
+      if (32 * s2 < D) {
+        bf16x8 ka, kb;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ka[j] = kb[j] = (bf16)0.f;
+        if (d0 + 8 <= D) {
+          ka = *reinterpret_cast<const bf16x8*>(r1 + d0);
+          kb = *reinterpret_cast<const bf16x8*>(r2 + d0);
+        }
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[s2], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qf[s2], s1, 0, 0, 0);
+      }
+    }
+    // the V^T pieces of this lane: 8 keys from k0 + 8 grp (clamped to the last piece that exists)
+    const int kp8 = min(k0 + 8 * grp, pos & ~7);
+    const bf16* vbase = v_cache + ((size_t)bt[kp8 / bs] * G + g) * Dv * bs + kp8 % bs;
+    float p[8];
+    float cm = -INFINITY;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int kp = k0 + 8 * grp + i;
+      const float sv = (i < 4 ? s0[i] : s1[i - 4]) * scale;
+      p[i] = (kp >= lo && kp <= pos) ? sv : -INFINITY;
+      cm = fmaxf(cm, p[i]);
+    }
+    cm = rows_max(cm);
+    const float m_new = fmaxf(m, cm);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;
+    const float alpha = m == -INFINITY ? 0.f : expf(m - m_new);
+    float ps = 0.f;
+    bf16x8 ph, pl;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float e = expf(p[i] - m_use);
+      ps += e;
+      ph[i] = (bf16)e;
+      pl[i] = (bf16)(e - (float)ph[i]);
+    }
+    l = l * alpha + rows_sum(ps);
+    m = m_new;
+#pragma unroll
+    for (int dt = 0; dt < NDV; ++dt) {
+      if (16 * dt < Dv) {
+        const int ch = 16 * dt + col;
+        bf16x8 va;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) va[j] = (bf16)0.f;
+        if (ch < Dv) va = *reinterpret_cast<const bf16x8*>(vbase + (size_t)ch * bs);
+        f32x4 a = acc[dt] * alpha;
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, ph, a, 0, 0, 0);
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl, a, 0, 0, 0);
+      }
+    }
+  }
+  // partial results: lane (col, grp) holds channels 16 dt + 4 grp + i of head col
+  if (grp == 0) sml[wave][0][col] = m, sml[wave][1][col] = l;
+#pragma unroll
+  for (int dt = 0; dt < NDV; ++dt)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) so[wave][col][16 * dt + 4 * grp + i] = acc[dt][i];
+  __syncthreads();
+  for (int idx = tid; idx < R * Dv; idx += 64 * kDW) {
+    const int hh = idx / Dv, e = idx - hh * Dv;
+    float mm = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < kDW; ++w) mm = fmaxf(mm, sml[w][0][hh]);
+    float ll = 0.f, o = 0.f;
+#pragma unroll
+    for (int w = 0; w < kDW; ++w) {
+      const float f = sml[w][0][hh] == -INFINITY ? 0.f : expf(sml[w][0][hh] - mm);
+      ll += sml[w][1][hh] * f;
+      o += so[w][hh][e] * f;
+    }
+    out[((size_t)t * H + g * R + hh) * Dv + e] = (bf16)(o / ll);
+  }
+}
+
+template <int NQK, int NDV>
+static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
+                          int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
+                          int Dv, int bs, int window, float scale, uintptr_t stream) {
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_decode_kernel<NQK, NDV>), dim3(rows, G), dim3(64 * kDW), 0,
+                     (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
+                     (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, H, G,
+                     D, Dv, bs, window, scale);
+  DLLM_HIP_CHECK(hipGetLastError());
+}
+
+// bf16 with 16-byte rows and pieces goes to the matrix cores; float32 (the exact path), odd head sizes
+// and heads wider than 256 take the row kernel
+static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs) {
+  return !f32 && D % 8 == 0 && Dv % 8 == 0 && bs % 8 == 0 && D <= 256 && Dv <= 256 && G > 0 && H % G == 0;
+}
+
 // Decode rows: tokens [0, rows) are one-token sequences.
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
                            int Dv, int bs, int window, float scale, int f32, uintptr_t stream) {
   if (rows <= 0) return;
+  if (win_mfma_ok(f32, H, G, D, Dv, bs) && H / G <= 16 && G <= 65535) {
+    DLLM_HOST_CHECK(window >= 1 && max_blocks > 0, "window attention sizes");
+#define WIN_DEC(NQK, NDV)                                                                                       \
+  launch_decode<NQK, NDV>(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, rows, H, G, D, Dv, \
+                          bs, window, scale, stream)
+    if (D <= 64 && Dv <= 64) WIN_DEC(2, 4);
+    else if (D <= 128 && Dv <= 128) WIN_DEC(4, 8);
+    else WIN_DEC(8, 16);
+#undef WIN_DEC
+    return;
+  }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, 0, rows, H, G, D, Dv, bs, window,
               scale, f32, stream);
 }
@@ -178,6 +491,18 @@ void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintp
   // tokens of the decode rows come first: one per sequence before seq0
   const int t0 = seq0;
   if (tokens <= t0) return;
+  if (win_mfma_ok(f32, H, G, D, Dv, bs) && seqs > seq0 && max_q_len > 1) {
+    DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && H <= 65535 && seqs - seq0 <= 65535, "window attention heads");
+    DLLM_HOST_CHECK(bs > 0 && window >= 1 && max_blocks > 0, "window attention sizes");
+#define WIN_TILE(NQK, NDV)                                                                                  \
+  launch_tile<NQK, NDV>(out, q, k_cache, v_cache, block_tables, max_blocks, cu, positions, seq0, seqs - seq0, \
+                        max_q_len, H, G, D, Dv, bs, window, scale, stream)
+    if (D <= 64 && Dv <= 64) WIN_TILE(2, 4);
+    else if (D <= 128 && Dv <= 128) WIN_TILE(4, 8);
+    else WIN_TILE(8, 16);
+#undef WIN_TILE
+    return;
+  }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, t0, tokens - t0, H, G, D, Dv, bs,
               window, scale, f32, stream);
 }

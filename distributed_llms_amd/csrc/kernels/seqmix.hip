@@ -369,7 +369,8 @@ void sm_softcap(uintptr_t out, uintptr_t x, long n, float cap, int f32, uintptr_
 // One wave per (token, head) of the fused projection [q heads | k heads | v heads]: the causal
 // convolution of the head's channels, then for q / k the RMS norm over the head (plain weight) and
 // the rotation of pairs (2i, 2i + 1), i < nrot, by pos * freqs[i] (cos and sin scaled by mag);
-// q goes to q_out [T, H, D], k / v to the paged caches [NB, G, BS, D] / [NB, G, BS, Dv].
+// q goes to q_out [T, H, D], k / v to the paged caches [NB, G, BS, D] / [NB, G, Dv, BS] (V transposed
+// inside a block).
 template <typename T>
 __global__ void __launch_bounds__(64) sm_attn_prep_kernel(
     void* __restrict__ q_out_, const void* __restrict__ qkv_, const void* __restrict__ conv_w_,
@@ -406,10 +407,10 @@ __global__ void __launch_bounds__(64) sm_attn_prep_kernel(
     const int slot = slot_mapping[t];
     const int blk = slot / bs, off = slot - blk * bs;
     if (kind == 1) dst = (T*)k_cache_ + (((size_t)blk * G + (head - H)) * bs + off) * D;
-    else dst = (T*)v_cache_ + (((size_t)blk * G + (head - H - G)) * bs + off) * Dv;
+    else dst = (T*)v_cache_ + ((size_t)blk * G + (head - H - G)) * Dv * bs + off;
   }
   if (kind == 2) {
-    for (int e = lane; e < n; e += 64) stf(dst + e, hv[e]);
+    for (int e = lane; e < n; e += 64) stf(dst + (size_t)e * bs, hv[e]);
     return;
   }
   ss = wave_sum(ss);

@@ -18,7 +18,7 @@ from .replay import TraceReplayer
 
 # name -> (width, layers, ff, heads, kv_heads, head size, rglru blocks, window)
 SIZES = {
-    "2b": (2560, 6, 7680, 20, 4, 128, 10, 2048),
+    "2b": (2560, 6, 7680, 16, 4, 128, 10, 2048),
     "9b": (4096, 6, 12288, 32, 8, 128, 16, 2048),
     "small": (1024, 6, 3072, 8, 2, 128, 4, 512),
 }
@@ -84,13 +84,17 @@ def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps:
 
 
 def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int = 32, reps: int = 2,
-        tmp: str = "/tmp/dllm_hybrid_bench") -> dict:
+        tmp: str = "/tmp/dllm_hybrid_bench", models=("tudilix", "llama")) -> dict:
     out = {"size": size, "batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
            "data": "synthetic (random-init weights, random token ids)"}
     for key, cfg, graphs in (("tudilix", hybrid_config(size), False), ("llama", llama_config(size), True)):
+        if key not in models:
+            continue
         p, d = _measure(cfg, batch, prompt_len, gen_len, reps, f"{tmp}/{key}", graphs)
         out[key] = {"prefill_tok_s": round(p, 1), "decode_tok_s": round(d, 1),
                     "params_m": round(cfg.param_count() / 1e6, 1)}
+    if len(models) < 2:
+        return out
     out["prefill_ratio"] = round(out["tudilix"]["prefill_tok_s"] / out["llama"]["prefill_tok_s"], 3)
     out["decode_ratio"] = round(out["tudilix"]["decode_tok_s"] / out["llama"]["decode_tok_s"], 3)
     return out

@@ -229,12 +229,12 @@ class HybridStage:
 
     def allocate_kv(self, num_blocks: int, block_size: int):
         """Paged caches of the attention layers with K/V of their own: k [NB, G, BS, dim],
-        v [NB, G, BS, vdim]; a ``kv_from`` layer reads its source's pair."""
+        v [NB, G, vdim, BS] (transposed inside a block); a ``kv_from`` layer reads its source's pair."""
         caches = {}
         for i in self.kv_layers:
             m = self.specs[i]["mixer"]
             caches[i] = (torch.zeros(num_blocks, m["kv_heads"], block_size, m["dim"], dtype=self.dtype, device=self.device),
-                         torch.zeros(num_blocks, m["kv_heads"], block_size, m["vdim"], dtype=self.dtype, device=self.device))
+                         torch.zeros(num_blocks, m["kv_heads"], m["vdim"], block_size, dtype=self.dtype, device=self.device))
         self.kv = _PagedCaches(caches, num_blocks, block_size)
         return self.kv
 

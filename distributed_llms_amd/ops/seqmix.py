@@ -299,7 +299,8 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
     convolution on every channel (``conv_w`` [C, taps], tail in ``state`` [slots, taps - 1, C]), the
     per-head RMS norm of q and k (plain weight), the interleaved-pair rotation of their first
     2 len(freqs) dims, and the append of k [.., dim] and v [.., vdim] (convolved only) at
-    ``slot_mapping`` into caches [NB, kv_heads, BS, dim] / [NB, kv_heads, BS, vdim].  With
+    ``slot_mapping`` into caches k [NB, kv_heads, BS, dim] / v [NB, kv_heads, vdim, BS] (V transposed inside
+    a block: the keys of one value channel are contiguous, which is what the matrix cores read).  With
     ``k_cache`` None the projection holds q only (the layer reads another layer's K/V).
     Returns q [T, heads, dim]."""
     t, c = qkv.shape
@@ -321,7 +322,7 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
             bs = k_cache.shape[2]
             sm = slot_mapping.long()
             k_cache[sm // bs, :, sm % bs] = k.to(k_cache.dtype)
-            v_cache[sm // bs, :, sm % bs] = v.to(v_cache.dtype)
+            v_cache[sm // bs, :, :, sm % bs] = v.to(v_cache.dtype)
         return q
     _ck(qkv, "qkv")
     _ck(conv_w, "conv_w", qkv.dtype)
@@ -332,7 +333,7 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
     if own_kv:
         _ck(k_cache, "k_cache", qkv.dtype)
         _ck(v_cache, "v_cache", qkv.dtype)
-        if k_cache.shape[1:] != (kv_heads, k_cache.shape[2], dim) or v_cache.shape[1:] != (kv_heads, k_cache.shape[2], vdim):
+        if k_cache.shape[1:] != (kv_heads, k_cache.shape[2], dim) or v_cache.shape[1:] != (kv_heads, vdim, k_cache.shape[2]):
             raise ValueError("attn_prep: cache shape")
     if 2 * freqs.numel() > dim:
         raise ValueError("attn_prep: rotary dims exceed the head size")
@@ -351,12 +352,12 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
                      sb: SeqBatch, window: int, scale: float, num_decode: Optional[int] = None) -> torch.Tensor:
     """Softmax attention of every query token over the keys j of its own sequence with
     0 <= p - j < window (p the query's position), keys / values read through ``block_tables`` from
-    caches [NB, G, BS, dim] / [NB, G, BS, vdim]; query head h reads K/V head h // (H / G).
+    caches k [NB, G, BS, dim] / v [NB, G, vdim, BS]; query head h reads K/V head h // (H / G).
     Scores and weights are float32.  ``num_decode``: the first that many sequences are one-token
     rows (they take the decode kernel; None: every sequence is one); the rest are prompt chunks.
     Returns [T, H, vdim]."""
     t, h, d = q.shape
-    g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[3]
+    g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     if not q.is_cuda:
         out = torch.empty(t, h, dv, dtype=torch.float32)
         pos, seq = sb.positions.tolist(), sb.tok_seq.tolist()
@@ -367,7 +368,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             idx = torch.arange(lo, p + 1)
             blk = block_tables[seq[i]].long()[idx // bs]
             kk = k_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)     # [n, H, d]
-            vv = v_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)
+            vv = v_cache[blk, :, :, idx % bs].float().repeat_interleave(rep, 1)
             s = torch.einsum("hd,nhd->hn", q[i].float(), kk) * scale
             out[i] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
         return out.to(q.dtype)
@@ -375,7 +376,7 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _ck(k_cache, "k_cache", q.dtype)
     _ck(v_cache, "v_cache", q.dtype)
     _ck(block_tables, "block_tables", torch.int32)
-    if h % g or k_cache.shape[3] != d or window < 1:
+    if h % g or k_cache.shape[3] != d or v_cache.shape[3] != bs or window < 1:
         raise ValueError("window_attention: head / size mismatch")
     out = torch.empty(t, h, dv, dtype=q.dtype, device=q.device)
     nd = sb.num_seqs if num_decode is None else int(num_decode)

@@ -273,10 +273,10 @@ def _paged(k, v, bs, device, dtype, num_blocks, table):
     """Scatter per-position k [n, G, D] / v [n, G, Dv] into paged caches following ``table``."""
     n, g, d = k.shape
     kc = torch.zeros(num_blocks, g, bs, d, dtype=dtype)
-    vc = torch.zeros(num_blocks, g, bs, v.shape[2], dtype=dtype)
+    vc = torch.zeros(num_blocks, g, v.shape[2], bs, dtype=dtype)
     for j in range(n):
         kc[table[j // bs], :, j % bs] = k[j]
-        vc[table[j // bs], :, j % bs] = v[j]
+        vc[table[j // bs], :, :, j % bs] = v[j]
     return kc.to(device), vc.to(device)
 
 
@@ -438,3 +438,44 @@ def test_config_round_trip_and_registry(tmp_path):
         bad["layers"][2]["mixer"]["kv_from"] = 1      # not an attention layer
         make_stage(ModelConfig.from_hf_config(bad))
     assert get_model_config("tiny-tudilix").arch == "tudilix"
+
+
+@pytest.mark.parametrize("target", TARGETS)
+@pytest.mark.parametrize("shape", [(4, 1, 64, 80, 96, 32), (8, 2, 128, 128, 70, 32), (2, 2, 256, 256, 33, 16),
+                                   (3, 3, 40, 24, 500, 64), (6, 2, 72, 136, 64, 32)])
+def test_window_attention_shapes(target, shape):
+    """Head sizes on both sides of the kernels' tile sizes, three chunks of unequal length that start
+    at different positions of their sequences (one at 0, one far in), windows shorter and longer than
+    a chunk, several block sizes; every query against the oracle."""
+    device, dtype = _dev(target)
+    h, g, d, dv, window, bs = shape
+    rng = np.random.default_rng(h * d + window)
+    chunks = [(0, 70), (37, 3), (161, 131)]                 # (start position, tokens)
+    T = lambda a: torch.from_numpy(a.astype(np.float32)).to(dtype)
+    nblocks = 64
+    free = list(rng.permutation(np.arange(1, nblocks)))
+    kcs = torch.zeros(nblocks, g, bs, d, dtype=dtype)
+    vcs = torch.zeros(nblocks, g, dv, bs, dtype=dtype)
+    tables, qs, wants = [], [], []
+    for start, n in chunks:
+        total = start + n
+        k, v, q = T(rng.standard_normal((total, g, d))), T(rng.standard_normal((total, g, dv))), T(rng.standard_normal((total, h, d)))
+        table = [int(free.pop()) for _ in range(-(-total // bs))]
+        for j in range(total):
+            kcs[table[j // bs], :, j % bs] = k[j]
+            vcs[table[j // bs], :, :, j % bs] = v[j]
+        tables.append(table)
+        qs.append(q[start:])
+        f64 = lambda t: t.float().numpy().astype(np.float64)
+        wants.append(O.window_attention(f64(q), f64(k), f64(v), window, d ** -0.5)[start:])
+    mb = max(len(t) for t in tables)
+    bt = torch.tensor([t + [0] * (mb - len(t)) for t in tables], dtype=torch.int32, device=device)
+    o = sm.window_attention(torch.cat(qs).contiguous().to(device), kcs.to(device), vcs.to(device), bt, _sb(chunks, device),
+                            window, d ** -0.5, num_decode=0)
+    t = 2e-5 if dtype == torch.float32 else 2e-2
+    np.testing.assert_allclose(o.float().cpu().numpy(), np.concatenate(wants), rtol=t, atol=t)
+    # the last token of every chunk once more, as one-token rows (the decode kernel)
+    rows = _sb([(s + n - 1, 1) for s, n in chunks], device)
+    qd = torch.stack([x[-1] for x in qs]).contiguous().to(device)
+    o = sm.window_attention(qd, kcs.to(device), vcs.to(device), bt, rows, window, d ** -0.5)
+    np.testing.assert_allclose(o.float().cpu().numpy(), np.stack([w[-1] for w in wants]), rtol=t, atol=t)
