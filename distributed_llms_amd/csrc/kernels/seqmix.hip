@@ -18,6 +18,49 @@ namespace dllm {
 template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
 template <typename T> __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
 
+// V consecutive elements <-> float registers: V = 8 moves 16 bytes of bf16 (32 of float) per lane and
+// needs the address aligned to 8 elements; V = 1 is the any-size form.
+template <int V> __device__ __forceinline__ void ldv(const bf16* p, float (&o)[V]) {
+  if constexpr (V == 8) {
+    const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) o[j] = bf2f(v[j]);
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) o[j] = bf2f(p[j]);
+  }
+}
+template <int V> __device__ __forceinline__ void ldv(const float* p, float (&o)[V]) {
+  if constexpr (V == 8) {
+    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) o[j] = a[j], o[4 + j] = b[j];
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) o[j] = p[j];
+  }
+}
+template <int V> __device__ __forceinline__ void stv(bf16* p, const float (&o)[V]) {
+  if constexpr (V == 8) {
+    bf16x8 v;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = f2bf(o[j]);
+    *reinterpret_cast<bf16x8*>(p) = v;
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) p[j] = f2bf(o[j]);
+  }
+}
+template <int V> __device__ __forceinline__ void stv(float* p, const float (&o)[V]) {
+  if constexpr (V == 8) {
+    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
+    *reinterpret_cast<f32x4*>(p + 4) = f32x4{o[4], o[5], o[6], o[7]};
+  } else {
+#pragma unroll
+    for (int j = 0; j < V; ++j) p[j] = o[j];
+  }
+}
+
 #define SM_DISPATCH(f32, KERNEL, grid, block, lds, stream, ...)                                        \
   do {                                                                                                 \
     if (f32)                                                                                           \
@@ -48,8 +91,8 @@ void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int
 }
 
 // --------------------------------------------------------------------------- RMS norm of an f32 row
-// y = x * rsqrt(mean(x^2) + eps) * (offset + w); one workgroup per row.
-template <typename T>
+// y = x * rsqrt(mean(x^2) + eps) * (offset + w); one workgroup per row, V elements per lane and step.
+template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_rms_norm_kernel(void* __restrict__ y_, const float* __restrict__ x,
                                                           const void* __restrict__ w_, int width, float eps,
                                                           float offset) {
@@ -58,26 +101,48 @@ __global__ void __launch_bounds__(256) sm_rms_norm_kernel(void* __restrict__ y_,
   const T* w = (const T*)w_;
   const float* xr = x + (size_t)blockIdx.x * width;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += 256) {
-    const float v = xr[i];
-    ss += v * v;
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+    float v[V];
+    ldv<V>(xr + i, v);
+#pragma unroll
+    for (int j = 0; j < V; ++j) ss += v[j] * v[j];
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
-  for (int i = threadIdx.x; i < width; i += 256) stf(y + i, xr[i] * inv * (offset + ldf(w + i)));
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+    float v[V], g[V];
+    ldv<V>(xr + i, v);
+    ldv<V>(w + i, g);
+#pragma unroll
+    for (int j = 0; j < V; ++j) v[j] = v[j] * inv * (offset + g[j]);
+    stv<V>(y + i, v);
+  }
 }
+
+#define SM_DISPATCH_V(f32, vec, KERNEL, grid, block, lds, stream, ...)                                          \
+  do {                                                                                                          \
+    hipStream_t s_ = (hipStream_t)(stream);                                                                     \
+    if (f32) {                                                                                                  \
+      if (vec) hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<float, 8>), grid, block, lds, s_, __VA_ARGS__);        \
+      else hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<float, 1>), grid, block, lds, s_, __VA_ARGS__);            \
+    } else {                                                                                                    \
+      if (vec) hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<bf16, 8>), grid, block, lds, s_, __VA_ARGS__);         \
+      else hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<bf16, 1>), grid, block, lds, s_, __VA_ARGS__);             \
+    }                                                                                                           \
+    DLLM_HIP_CHECK(hipGetLastError());                                                                          \
+  } while (0)
 
 void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, float eps, float offset, int f32,
                  uintptr_t stream) {
   if (rows <= 0) return;
   DLLM_HOST_CHECK(width > 0, "norm width");
-  SM_DISPATCH(f32, sm_rms_norm_kernel, dim3(rows), dim3(256), 0, stream, (void*)y, (const float*)x, (const void*)w,
-              width, eps, offset);
+  SM_DISPATCH_V(f32, width % 8 == 0, sm_rms_norm_kernel, dim3(rows), dim3(256), 0, stream, (void*)y, (const float*)x,
+                (const void*)w, width, eps, offset);
 }
 
 // --------------------------------------------------------------------------- close of a sublayer
 // x += mult * rms_norm(o + bias) * (1 + w_post);  h = rms_norm(x) * (1 + w_next) when w_next.
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict__ x, const void* __restrict__ o_,
                                                                const void* __restrict__ bias_,
                                                                const void* __restrict__ wp_,
@@ -90,47 +155,82 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
   const T* wn = (const T*)wn_;
   float* xr = x + (size_t)blockIdx.x * width;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < width; i += 256) {
-    const float v = ldf(o + i) + (bias ? ldf(bias + i) : 0.f);
-    ss += v * v;
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+    float v[V], bb[V];
+    ldv<V>(o + i, v);
+    if (bias) {
+      ldv<V>(bias + i, bb);
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] += bb[j];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) ss += v[j] * v[j];
   }
   ss = block_sum(ss, red);
   const float inv = 1.0f / sqrtf(ss / (float)width + eps);
   float s2 = 0.f;
-  for (int i = threadIdx.x; i < width; i += 256) {
-    const float v = ldf(o + i) + (bias ? ldf(bias + i) : 0.f);
-    const float nx = xr[i] + mult * (v * inv * (1.0f + ldf(wp + i)));
-    xr[i] = nx;
-    s2 += nx * nx;
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {
+    float v[V], bb[V], g[V], xv[V];
+    ldv<V>(o + i, v);
+    if (bias) {
+      ldv<V>(bias + i, bb);
+#pragma unroll
+      for (int j = 0; j < V; ++j) v[j] += bb[j];
+    }
+    ldv<V>(wp + i, g);
+    ldv<V>(xr + i, xv);
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      xv[j] = xv[j] + mult * (v[j] * inv * (1.0f + g[j]));
+      s2 += xv[j] * xv[j];
+    }
+    stv<V>(xr + i, xv);
   }
   if (!wn) return;
   s2 = block_sum(s2, red);
   const float inv2 = 1.0f / sqrtf(s2 / (float)width + eps);
   T* h = (T*)h_ + (size_t)blockIdx.x * width;
-  for (int i = threadIdx.x; i < width; i += 256) stf(h + i, xr[i] * inv2 * (1.0f + ldf(wn + i)));
+  for (int i = threadIdx.x * V; i < width; i += 256 * V) {      // each lane re-reads what it wrote itself
+    float xv[V], g[V];
+    ldv<V>(xr + i, xv);
+    ldv<V>(wn + i, g);
+#pragma unroll
+    for (int j = 0; j < V; ++j) xv[j] = xv[j] * inv2 * (1.0f + g[j]);
+    stv<V>(h + i, xv);
+  }
 }
 
 void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
                       int rows, int width, float eps, float mult, int f32, uintptr_t stream) {
   if (rows <= 0) return;
   DLLM_HOST_CHECK(width > 0 && (!w_next || h), "post_norm_add arguments");
-  SM_DISPATCH(f32, sm_post_norm_add_kernel, dim3(rows), dim3(256), 0, stream, (float*)x, (const void*)o,
-              (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult);
+  SM_DISPATCH_V(f32, width % 8 == 0, sm_post_norm_add_kernel, dim3(rows), dim3(256), 0, stream, (float*)x,
+                (const void*)o, (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult);
 }
 
 // --------------------------------------------------------------------------- causal convolution with state
 // Input d rows before token (t, channel c) of a chunk that starts at position `start` with the token
 // at local index tl: the batch row t - d while tl - d >= 0, else the state tail row
 // tl - d + (taps - 1) while the position start + tl - d >= 0, else zero (before the sequence).
+// Weights are stored [taps, C] (tap-major), so V consecutive channels of one tap are one load.
 template <typename T>
 __device__ __forceinline__ float conv_input(const T* __restrict__ u, long stride, const T* __restrict__ st, int t,
-                                            int tl, int pos, int d, int taps, int c, int C, float in_bias) {
+                                            int tl, int pos, int d, int taps, int c, int C) {
   if (d > pos) return 0.f;
-  if (d <= tl) return ldf(u + (size_t)(t - d) * stride + c) + in_bias;
-  return ldf(st + (size_t)(tl - d + taps - 1) * C + c) + in_bias;
+  if (d <= tl) return ldf(u + (size_t)(t - d) * stride + c);
+  return ldf(st + (size_t)(tl - d + taps - 1) * C + c);
 }
 
-template <typename T, typename OT>
+template <typename T, int V>
+__device__ __forceinline__ bool conv_input_v(const T* __restrict__ u, long stride, const T* __restrict__ st, int t,
+                                             int tl, int pos, int d, int taps, int c, int C, float (&o)[V]) {
+  if (d > pos) return false;
+  if (d <= tl) ldv<V>(u + (size_t)(t - d) * stride + c, o);
+  else ldv<V>(st + (size_t)(tl - d + taps - 1) * C + c, o);
+  return true;
+}
+
+template <typename T, typename OT, int V>
 __global__ void __launch_bounds__(256) sm_causal_conv_kernel(void* __restrict__ y_, const void* __restrict__ u_,
                                                              long stride, const void* __restrict__ w_,
                                                              const void* __restrict__ bias_,
@@ -149,19 +249,26 @@ __global__ void __launch_bounds__(256) sm_causal_conv_kernel(void* __restrict__ 
   const T* bias = (const T*)bias_;
   const T* in_bias = (const T*)in_bias_;
   OT* y = (OT*)y_ + (size_t)t * C;
-  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
-    const float ib = in_bias ? ldf(in_bias + c) : 0.f;
-    float acc = bias ? ldf(bias + c) : 0.f;
-    for (int j = 0; j < taps; ++j)
-      acc += ldf(w + (size_t)c * taps + j) * conv_input(u, stride, st, t, tl, pos, taps - 1 - j, taps, c, C, ib);
-    stf(y + c, acc);
+  for (int c = (blockIdx.y * 256 + threadIdx.x) * V; c < C; c += gridDim.y * 256 * V) {
+    float acc[V], ib[V], xv[V], wv[V];
+#pragma unroll
+    for (int j = 0; j < V; ++j) acc[j] = 0.f, ib[j] = 0.f;
+    if (bias) ldv<V>(bias + c, acc);
+    if (in_bias) ldv<V>(in_bias + c, ib);
+    for (int j = 0; j < taps; ++j) {
+      if (!conv_input_v<T, V>(u, stride, st, t, tl, pos, taps - 1 - j, taps, c, C, xv)) continue;
+      ldv<V>(w + (size_t)j * C + c, wv);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += wv[e] * (xv[e] + ib[e]);
+    }
+    stv<V>(y + c, acc);
   }
 }
 
 // New tail of every sequence: row j of the state becomes the input at position end - (taps - 1) + j
-// (end = the chunk's last position + 1).  One thread per (sequence, channel) walks j upwards: row j
+// (end = the chunk's last position + 1).  One thread per (sequence, V channels) walks j upwards: row j
 // of the old tail is read (as row j + n, n the chunk's length) only before it is overwritten.
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_conv_state_kernel(void* __restrict__ state_, const void* __restrict__ u_,
                                                             long stride, const int32_t* __restrict__ cu,
                                                             const int32_t* __restrict__ positions,
@@ -172,16 +279,25 @@ __global__ void __launch_bounds__(256) sm_conv_state_kernel(void* __restrict__ s
   const int start = positions[lo];
   T* st = (T*)state_ + (size_t)slots[b] * (taps - 1) * C;
   const T* u = (const T*)u_;
-  for (int c = blockIdx.y * 256 + threadIdx.x; c < C; c += gridDim.y * 256) {
+  for (int c = (blockIdx.y * 256 + threadIdx.x) * V; c < C; c += gridDim.y * 256 * V) {
     for (int j = 0; j < taps - 1; ++j) {
       const int tl = n - (taps - 1) + j;              // local index of the row that lands in tail row j
-      float v;
-      if (tl >= 0) v = ldf(u + (size_t)(lo + tl) * stride + c);
-      else if (start + tl >= 0) v = ldf(st + (size_t)(j + n) * C + c);
-      else v = 0.f;
-      stf(st + (size_t)j * C + c, v);
+      float v[V];
+#pragma unroll
+      for (int e = 0; e < V; ++e) v[e] = 0.f;
+      if (tl >= 0) ldv<V>(u + (size_t)(lo + tl) * stride + c, v);
+      else if (start + tl >= 0) ldv<V>(st + (size_t)(j + n) * C + c, v);
+      stv<V>(st + (size_t)j * C + c, v);
     }
   }
+}
+
+static void launch_conv_state(uintptr_t state, uintptr_t u, long stride, uintptr_t cu, uintptr_t positions,
+                              uintptr_t slots, int seqs, int C, int taps, int f32, int vec, uintptr_t stream) {
+  const int per = 256 * (vec ? 8 : 1);
+  SM_DISPATCH_V(f32, vec, sm_conv_state_kernel, dim3(seqs, std::min(8, (C + per - 1) / per)), dim3(256), 0, stream,
+                (void*)state, (const void*)u, stride, (const int32_t*)cu, (const int32_t*)positions,
+                (const int32_t*)slots, C, taps);
 }
 
 void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,
@@ -189,47 +305,48 @@ void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_
                     int tokens, int seqs, int C, int taps, int f32, int out_f32, uintptr_t stream) {
   if (tokens <= 0 || seqs <= 0) return;
   DLLM_HOST_CHECK(C > 0 && taps >= 1 && stride >= C, "conv sizes");
-  const dim3 grid(tokens, std::min(8, (C + 255) / 256));
+  const int esz = f32 ? 4 : 2;
+  const int vec = C % 8 == 0 && stride % 8 == 0 && (u % (8 * esz)) == 0;
+  const int per = 256 * (vec ? 8 : 1);
+  const dim3 grid(tokens, std::min(8, (C + per - 1) / per));
   hipStream_t s = (hipStream_t)stream;
-#define SM_CONV(T, OT)                                                                                       \
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(sm_causal_conv_kernel<T, OT>), grid, dim3(256), 0, s, (void*)y, (const void*)u, \
+#define SM_CONV(T, OT, V)                                                                                    \
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(sm_causal_conv_kernel<T, OT, V>), grid, dim3(256), 0, s, (void*)y, (const void*)u, \
                      stride, (const void*)w, (const void*)bias, (const void*)in_bias, (const void*)state,     \
                      (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots, C, taps)
-  if (f32) SM_CONV(float, float);
-  else if (out_f32) SM_CONV(bf16, float);
-  else SM_CONV(bf16, bf16);
+  if (f32) { if (vec) SM_CONV(float, float, 8); else SM_CONV(float, float, 1); }
+  else if (out_f32) { if (vec) SM_CONV(bf16, float, 8); else SM_CONV(bf16, float, 1); }
+  else { if (vec) SM_CONV(bf16, bf16, 8); else SM_CONV(bf16, bf16, 1); }
 #undef SM_CONV
   DLLM_HIP_CHECK(hipGetLastError());
-  if (taps > 1)
-    SM_DISPATCH(f32, sm_conv_state_kernel, dim3(seqs, std::min(8, (C + 255) / 256)), dim3(256), 0, stream,
-                (void*)state, (const void*)u, stride, (const int32_t*)cu, (const int32_t*)positions,
-                (const int32_t*)slots, C, taps);
+  if (taps > 1) launch_conv_state(state, u, stride, cu, positions, slots, seqs, C, taps, f32, vec, stream);
 }
 
 // --------------------------------------------------------------------------- RG-LRU gates
-// a = exp(-scale * sigmoid(Ra_b u_b + ra_b) * softplus(lam)),  g = sqrt(1 - a^2) * sigmoid(Ri_b u_b + ri_b) * u
-// for GT tokens x one block of bw channels per workgroup; the token tile's u_b sits in LDS, the
-// transposed gate matrices [nb, in, out] are read with consecutive lanes on consecutive outputs.
-constexpr int GT = 8;
-
+// a = exp(-scale * sigmoid(Ra_b u_b + ra_b) * softplus(lam)),  g = sqrt(1 - a^2) * sigmoid(Ri_b u_b + ri_b) * u,
+// with the transposed gate matrices [nb, in, out] (consecutive lanes on consecutive outputs).
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 __device__ __forceinline__ float softplus_f(float x) { return fmaxf(x, 0.f) + log1pf(expf(-fabsf(x))); }
 
+// Few tokens (decode): GT tokens x one block of bw channels per workgroup on the vector ALUs; the
+// token tile's u_b sits in LDS, every weight is read once per workgroup.
+constexpr int GT = 4;
+
 template <typename T>
-__global__ void __launch_bounds__(256) sm_rglru_gates_kernel(float* __restrict__ a_out, float* __restrict__ g_out,
-                                                             const float* __restrict__ u,
-                                                             const void* __restrict__ ra_t_,
-                                                             const void* __restrict__ ra_b_,
-                                                             const void* __restrict__ ri_t_,
-                                                             const void* __restrict__ ri_b_,
-                                                             const void* __restrict__ lam_, int tokens, int nb, int bw,
-                                                             float scale) {
-  extern __shared__ float ub[];                       // [GT][bw]
+__global__ void __launch_bounds__(256) sm_rglru_gates_small_kernel(float* __restrict__ a_out, float* __restrict__ g_out,
+                                                                   const float* __restrict__ u,
+                                                                   const void* __restrict__ ra_t_,
+                                                                   const void* __restrict__ ra_b_,
+                                                                   const void* __restrict__ ri_t_,
+                                                                   const void* __restrict__ ri_b_,
+                                                                   const void* __restrict__ lam_, int tokens, int nb,
+                                                                   int bw, float scale) {
+  extern __shared__ float ubs[];                      // [GT][bw]
   const int t0 = blockIdx.x * GT, b = blockIdx.y, C = nb * bw;
   const int nt = min(GT, tokens - t0);
   for (int i = threadIdx.x; i < GT * bw; i += 256) {
     const int k = i / bw, c = i - k * bw;
-    ub[i] = k < nt ? u[(size_t)(t0 + k) * C + b * bw + c] : 0.f;
+    ubs[i] = k < nt ? u[(size_t)(t0 + k) * C + b * bw + c] : 0.f;
   }
   __syncthreads();
   const T* ra = (const T*)ra_t_ + (size_t)b * bw * bw;
@@ -239,11 +356,26 @@ __global__ void __launch_bounds__(256) sm_rglru_gates_kernel(float* __restrict__
     const float br = ldf((const T*)ra_b_ + b * bw + o), bi = ldf((const T*)ri_b_ + b * bw + o);
 #pragma unroll
     for (int k = 0; k < GT; ++k) ar[k] = br, ai[k] = bi;
-    for (int i = 0; i < bw; ++i) {
+    int i = 0;
+    for (; i + 8 <= bw; i += 8) {                      // 16 weight loads in flight, then their FMAs
+      float wr[8], wi[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) wr[j] = ldf(ra + (size_t)(i + j) * bw + o), wi[j] = ldf(ri + (size_t)(i + j) * bw + o);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+#pragma unroll
+        for (int k = 0; k < GT; ++k) {
+          const float x = ubs[k * bw + i + j];
+          ar[k] = fmaf(wr[j], x, ar[k]);
+          ai[k] = fmaf(wi[j], x, ai[k]);
+        }
+      }
+    }
+    for (; i < bw; ++i) {
       const float wr = ldf(ra + (size_t)i * bw + o), wi = ldf(ri + (size_t)i * bw + o);
 #pragma unroll
       for (int k = 0; k < GT; ++k) {
-        const float x = ub[k * bw + i];
+        const float x = ubs[k * bw + i];
         ar[k] = fmaf(wr, x, ar[k]);
         ai[k] = fmaf(wi, x, ai[k]);
       }
@@ -255,7 +387,87 @@ __global__ void __launch_bounds__(256) sm_rglru_gates_kernel(float* __restrict__
         const float av = expf(-scale * sigmoid_f(ar[k]) * sp);
         const size_t idx = (size_t)(t0 + k) * C + b * bw + o;
         a_out[idx] = av;
-        g_out[idx] = sqrtf(1.0f - av * av) * sigmoid_f(ai[k]) * ub[k * bw + o];
+        g_out[idx] = sqrtf(1.0f - av * av) * sigmoid_f(ai[k]) * ubs[k * bw + o];
+      }
+    }
+  }
+}
+
+// Many tokens (prompts): the two block-diagonal products on the float32 matrix cores
+// (v_mfma_f32_32x32x2_f32: true 32-bit operands and sums, which the gates of the recurrence require).
+// One workgroup per (64 tokens, block b, 128 outputs of the block): each wave owns 32 outputs and, for
+// both gates, two 32 x 32 accumulators (token rows 0-31 and 32-63).  The token tile's u_b passes through
+// LDS in K chunks of kGK (A operand: lane l = row l % 32, k l / 32); the gate matrices are the B operand
+// from global memory, kGU k-steps of loads issued ahead of the MFMAs that use them.
+constexpr int kGT = 64;       // tokens per workgroup
+constexpr int kGK = 128;      // K chunk in LDS
+constexpr int kGU = 8;        // k-steps (of 2) per group of loads
+
+template <typename T>
+__global__ void __launch_bounds__(256) sm_rglru_gates_kernel(float* __restrict__ a_out, float* __restrict__ g_out,
+                                                             const float* __restrict__ u,
+                                                             const void* __restrict__ ra_t_,
+                                                             const void* __restrict__ ra_b_,
+                                                             const void* __restrict__ ri_t_,
+                                                             const void* __restrict__ ri_b_,
+                                                             const void* __restrict__ lam_, int tokens, int nb, int bw,
+                                                             float scale) {
+  __shared__ float ub[kGT][kGK + 1];
+  const int t0 = blockIdx.x * kGT, b = blockIdx.y, C = nb * bw;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, n = lane & 31, half = lane >> 5;
+  const int o = blockIdx.z * 128 + wave * 32 + n;            // this lane's output channel inside block b
+  const int oc = min(o, bw - 1);
+  const T* ra = (const T*)ra_t_ + (size_t)b * bw * bw;
+  const T* ri = (const T*)ri_t_ + (size_t)b * bw * bw;
+  f32x16 cr0, ci0, cr1, ci1;
+#pragma unroll
+  for (int i = 0; i < 16; ++i) cr0[i] = ci0[i] = cr1[i] = ci1[i] = 0.f;
+  for (int kc = 0; kc < bw; kc += kGK) {
+    const int kn = min(kGK, bw - kc);
+    __syncthreads();
+    for (int i = tid; i < kGT * kGK; i += 256) {
+      const int r = i / kGK, k = i - r * kGK;
+      ub[r][k] = (t0 + r < tokens && k < kn) ? u[(size_t)(t0 + r) * C + b * bw + kc + k] : 0.f;
+    }
+    __syncthreads();
+    for (int ks0 = 0; 2 * ks0 < kn; ks0 += kGU) {
+      float br[kGU], bi[kGU], a0[kGU], a1[kGU];
+#pragma unroll
+      for (int j = 0; j < kGU; ++j) {
+        const int k = 2 * (ks0 + j) + half;                  // inside the chunk
+        const bool ok = k < kn && o < bw;
+        const size_t at = (size_t)(kc + min(k, kn - 1)) * bw + oc;
+        const float wr = ldf(ra + at), wi = ldf(ri + at);
+        br[j] = ok ? wr : 0.f;
+        bi[j] = ok ? wi : 0.f;
+        const int kk = min(k, kGK - 1);
+        a0[j] = k < kn ? ub[n][kk] : 0.f;
+        a1[j] = k < kn ? ub[32 + n][kk] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < kGU; ++j) {
+        cr0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[j], br[j], cr0, 0, 0, 0);
+        ci0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[j], bi[j], ci0, 0, 0, 0);
+        cr1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], br[j], cr1, 0, 0, 0);
+        ci1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], bi[j], ci1, 0, 0, 0);
+      }
+    }
+  }
+  if (o >= bw) return;
+  const int ch = b * bw + o;
+  const float rb = ldf((const T*)ra_b_ + ch), ib = ldf((const T*)ri_b_ + ch);
+  const float sp = softplus_f(ldf((const T*)lam_ + ch));
+#pragma unroll
+  for (int hh = 0; hh < 2; ++hh) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      const int row = 32 * hh + 8 * (i >> 2) + 4 * half + (i & 3);    // accumulator register i of this lane
+      const int t = t0 + row;
+      if (t < tokens) {
+        const float av = expf(-scale * sigmoid_f((hh ? cr1[i] : cr0[i]) + rb) * sp);
+        const size_t idx = (size_t)t * C + ch;
+        a_out[idx] = av;
+        g_out[idx] = sqrtf(1.0f - av * av) * sigmoid_f((hh ? ci1[i] : ci0[i]) + ib) * u[idx];
       }
     }
   }
@@ -265,17 +477,17 @@ void sm_rglru_gates(uintptr_t a, uintptr_t g, uintptr_t u, uintptr_t ra_t, uintp
                     uintptr_t ri_b, uintptr_t lam, int tokens, int nb, int bw, float scale, int f32,
                     uintptr_t stream) {
   if (tokens <= 0) return;
-  DLLM_HOST_CHECK(nb > 0 && bw > 0 && (size_t)GT * bw * 4 <= 160 * 1024 && nb <= 65535, "rglru gate sizes");
+  DLLM_HOST_CHECK(nb > 0 && bw > 0 && nb <= 65535 && (bw + 127) / 128 <= 65535, "rglru gate sizes");
   const size_t lds = (size_t)GT * bw * sizeof(float);
-  if (lds > 48 * 1024) {
-    if (f32) DLLM_HIP_CHECK(hipFuncSetAttribute((const void*)sm_rglru_gates_kernel<float>,
-                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    else DLLM_HIP_CHECK(hipFuncSetAttribute((const void*)sm_rglru_gates_kernel<bf16>,
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  if (tokens <= 64 && lds <= 48 * 1024) {
+    SM_DISPATCH(f32, sm_rglru_gates_small_kernel, dim3((tokens + GT - 1) / GT, nb), dim3(256), lds, stream, (float*)a,
+                (float*)g, (const float*)u, (const void*)ra_t, (const void*)ra_b, (const void*)ri_t,
+                (const void*)ri_b, (const void*)lam, tokens, nb, bw, scale);
+    return;
   }
-  SM_DISPATCH(f32, sm_rglru_gates_kernel, dim3((tokens + GT - 1) / GT, nb), dim3(256), lds, stream, (float*)a,
-              (float*)g, (const float*)u, (const void*)ra_t, (const void*)ra_b, (const void*)ri_t, (const void*)ri_b,
-              (const void*)lam, tokens, nb, bw, scale);
+  SM_DISPATCH(f32, sm_rglru_gates_kernel, dim3((tokens + kGT - 1) / kGT, nb, (bw + 127) / 128), dim3(256), 0, stream,
+              (float*)a, (float*)g, (const float*)u, (const void*)ra_t, (const void*)ra_b, (const void*)ri_t,
+              (const void*)ri_b, (const void*)lam, tokens, nb, bw, scale);
 }
 
 // --------------------------------------------------------------------------- RG-LRU scan
@@ -302,7 +514,24 @@ __global__ void __launch_bounds__(64) sm_rglru_scan_kernel(void* __restrict__ ou
   float* sp = state + (size_t)slots[b] * C + c;
   float s = positions[lo] > 0 ? *sp : 0.f;
   const float yb = ldf((const T*)y_bias_ + c);
-  for (int t = lo; t < hi; ++t) {
+  // the recurrence is a dependent chain, its operands are not: 8 steps' loads go out together
+  int t = lo;
+  for (; t + 8 <= hi; t += 8) {
+    float av[8], gv[8], yv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const size_t i = (size_t)(t + j) * C + c;
+      av[j] = a[i];
+      gv[j] = g[i];
+      yv[j] = ldf(y_raw + (size_t)(t + j) * y_stride + c);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      s = fmaf(av[j], s, gv[j]);
+      stf(out + (size_t)(t + j) * C + c, s * gelu_tanh_f(yv[j] + yb));
+    }
+  }
+  for (; t < hi; ++t) {
     const size_t i = (size_t)t * C + c;
     s = fmaf(a[i], s, g[i]);
     stf(out + i, s * gelu_tanh_f(ldf(y_raw + (size_t)t * y_stride + c) + yb));
@@ -321,31 +550,39 @@ void sm_rglru_scan(uintptr_t out, uintptr_t a, uintptr_t g, uintptr_t y_raw, lon
 }
 
 // --------------------------------------------------------------------------- clipped GLU
-template <typename T>
+template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_clipped_glu_kernel(void* __restrict__ out_, const void* __restrict__ gu_,
-                                                             const void* __restrict__ bias_, long n, int F,
-                                                             float limit, float alpha) {
-  const T* gu = (const T*)gu_;
+                                                             const void* __restrict__ bias_, int F, float limit,
+                                                             float alpha) {
+  const T* gu = (const T*)gu_ + (size_t)blockIdx.x * 2 * F;
   const T* bias = (const T*)bias_;
-  T* out = (T*)out_;
-  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
-    const long t = i / F;
-    const int c = (int)(i - t * F);
-    float gv = ldf(gu + t * 2 * F + c), uv = ldf(gu + t * 2 * F + F + c);
-    if (bias) gv += ldf(bias + c), uv += ldf(bias + F + c);
-    gv = fminf(gv, limit);
-    uv = fminf(fmaxf(uv, -limit), limit);
-    stf(out + i, gv * (1.0f / (1.0f + expf(-alpha * gv))) * (uv + 1.0f));
+  T* out = (T*)out_ + (size_t)blockIdx.x * F;
+  for (int c = (blockIdx.y * 256 + threadIdx.x) * V; c < F; c += gridDim.y * 256 * V) {
+    float gv[V], uv[V], b1[V], b2[V];
+    ldv<V>(gu + c, gv);
+    ldv<V>(gu + F + c, uv);
+    if (bias) {
+      ldv<V>(bias + c, b1);
+      ldv<V>(bias + F + c, b2);
+#pragma unroll
+      for (int j = 0; j < V; ++j) gv[j] += b1[j], uv[j] += b2[j];
+    }
+#pragma unroll
+    for (int j = 0; j < V; ++j) {
+      const float g = fminf(gv[j], limit), u = fminf(fmaxf(uv[j], -limit), limit);
+      gv[j] = g * (1.0f / (1.0f + expf(-alpha * g))) * (u + 1.0f);
+    }
+    stv<V>(out + c, gv);
   }
 }
 
 void sm_clipped_glu(uintptr_t out, uintptr_t gu, uintptr_t bias, int tokens, int F, float limit, float alpha, int f32,
                     uintptr_t stream) {
-  const long n = (long)tokens * F;
-  if (n <= 0) return;
-  const int grid = (int)std::min<long>((n + 255) / 256, 65535);
-  SM_DISPATCH(f32, sm_clipped_glu_kernel, dim3(grid), dim3(256), 0, stream, (void*)out, (const void*)gu,
-              (const void*)bias, n, F, limit, alpha);
+  if (tokens <= 0 || F <= 0) return;
+  const int vec = F % 8 == 0;
+  const int per = 256 * (vec ? 8 : 1);
+  SM_DISPATCH_V(f32, vec, sm_clipped_glu_kernel, dim3(tokens, std::min(16, (F + per - 1) / per)), dim3(256), 0, stream,
+                (void*)out, (const void*)gu, (const void*)bias, F, limit, alpha);
 }
 
 // --------------------------------------------------------------------------- logit soft cap
@@ -397,7 +634,7 @@ __global__ void __launch_bounds__(64) sm_attn_prep_kernel(
     const int c = c0 + e;
     float acc = 0.f;
     for (int j = 0; j < taps; ++j)
-      acc += ldf(w + (size_t)c * taps + j) * conv_input(qkv, (long)C, st, t, tl, pos, taps - 1 - j, taps, c, C, 0.f);
+      acc += ldf(w + (size_t)j * C + c) * conv_input(qkv, (long)C, st, t, tl, pos, taps - 1 - j, taps, c, C);
     hv[e] = acc;
     ss += acc * acc;
   }
@@ -450,9 +687,7 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
               (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots, H, G, D, Dv, taps, bs);
   // the projection's last taps - 1 rows of every sequence become its new tail
   if (taps > 1)
-    SM_DISPATCH(f32, sm_conv_state_kernel, dim3(seqs, std::min(8, (C + 255) / 256)), dim3(256), 0, stream,
-                (void*)state, (const void*)qkv, (long)C, (const int32_t*)cu, (const int32_t*)positions,
-                (const int32_t*)slots, C, taps);
+    launch_conv_state(state, qkv, (long)C, cu, positions, slots, seqs, C, taps, f32, C % 8 == 0, stream);
 }
 
 }  // namespace dllm

@@ -166,7 +166,7 @@ class HybridStage:
 
     def load_hf_state(self, sd: Dict[str, torch.Tensor]) -> "HybridStage":
         """From checkpoint-named tensors: fuses y|x, q|k|v (and their convolutions), gate|up, and stores
-        the gate matrices transposed ([blocks, in, out])."""
+        the gate matrices transposed ([blocks, in, out]) and the convolution weights tap-major ([taps, C])."""
         want = model_shapes(self.cfg)
         for n, shp in want.items():
             if n not in sd:
@@ -184,13 +184,14 @@ class HybridStage:
             if layer["type"] == "attention":
                 parts = ["q"] if "kv_from" in layer["mixer"] else ["q", "k", "v"]
                 w["wqkv"] = cat([p + f"mix.{x}" for x in parts])
-                w["conv_w"] = cat([p + f"mix.{x}.conv" for x in parts])
+                w["conv_w"] = cv(torch.cat([sd[p + f"mix.{x}.conv"] for x in parts], 0).t())     # [taps, C]
                 w["q_norm"] = cv(sd[p + "mix.q.norm"])
                 if len(parts) == 3:
                     w["k_norm"] = cv(sd[p + "mix.k.norm"])
             else:
                 w["w_yx"] = cat([p + "mix.y", p + "mix.x"])
-                for k, n in (("y_b", "mix.y.b"), ("x_b", "mix.x.b"), ("conv_w", "mix.conv"), ("conv_b", "mix.conv.b"),
+                w["conv_w"] = cv(sd[p + "mix.conv"].t())                                        # [taps, C]
+                for k, n in (("y_b", "mix.y.b"), ("x_b", "mix.x.b"), ("conv_b", "mix.conv.b"),
                              ("ra_b", "mix.ra.b"), ("ri_b", "mix.ri.b"), ("lam", "mix.lam")):
                     w[k] = cv(sd[p + n])
                 w["ra_t"] = cv(sd[p + "mix.ra"].transpose(1, 2))

@@ -149,12 +149,12 @@ def causal_conv(u: torch.Tensor, w: torch.Tensor, bias: Optional[torch.Tensor], 
     (zeros before the sequence's start), across chunk borders: ``state`` [slots, taps - 1, C] holds each
     sequence's last taps - 1 rows of ``u`` and is brought up to date.  ``u`` [T, C] may be a column slice
     of a wider projection (row stride); ``in_bias`` is the bias of the projection that made it."""
-    c, taps = w.shape
+    taps, c = w.shape
     if u.shape[1] != c or state.shape[1:] != (taps - 1, c):
         raise ValueError("causal_conv: shape mismatch")
     if not u.is_cuda:
         g = _ref_conv_gather(u, state, sb, taps, in_bias)
-        y = (g * w.float().t()[:, None, :]).sum(0)
+        y = (g * w.float()[:, None, :]).sum(0)
         if bias is not None:
             y = y + bias.float()
         return y.to(out_dtype)
@@ -296,7 +296,7 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
               k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], slot_mapping: torch.Tensor,
               sb: SeqBatch, heads: int, kv_heads: int, dim: int, vdim: int) -> torch.Tensor:
     """From the fused projection [T, heads * dim (+ kv_heads * dim + kv_heads * vdim)]: the short causal
-    convolution on every channel (``conv_w`` [C, taps], tail in ``state`` [slots, taps - 1, C]), the
+    convolution on every channel (``conv_w`` [taps, C], tap-major; tail in ``state`` [slots, taps - 1, C]), the
     per-head RMS norm of q and k (plain weight), the interleaved-pair rotation of their first
     2 len(freqs) dims, and the append of k [.., dim] and v [.., vdim] (convolved only) at
     ``slot_mapping`` into caches k [NB, kv_heads, BS, dim] / v [NB, kv_heads, vdim, BS] (V transposed inside
@@ -306,12 +306,12 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
     t, c = qkv.shape
     own_kv = k_cache is not None
     qc, kc, vc = heads * dim, kv_heads * dim, kv_heads * vdim
-    if c != qc + (kc + vc if own_kv else 0) or conv_w.shape[0] != c:
+    if c != qc + (kc + vc if own_kv else 0) or conv_w.shape[1] != c:
         raise ValueError("attn_prep: projection width mismatch")
-    taps = conv_w.shape[1]
+    taps = conv_w.shape[0]
     if not qkv.is_cuda:
         g = _ref_conv_gather(qkv, state, sb, taps)
-        y = (g * conv_w.float().t()[:, None, :]).sum(0)
+        y = (g * conv_w.float()[:, None, :]).sum(0)
         pos = sb.positions
         q = _ref_rms(y[:, :qc].view(t, heads, dim), q_norm, eps, 0.0)
         q = _ref_rope_interleaved(q, pos, freqs, mag).to(qkv.dtype)

@@ -177,7 +177,7 @@ def test_causal_conv_across_portions(target, taps):
     read by a sequence that starts at 0."""
     device, dtype = _dev(target)
     rng = np.random.default_rng(taps)
-    c, n = 70, 23
+    c, n = (136 if taps == 4 else 70), 23          # 136: the 8-channel vector path, 70: the any-size path
     u = torch.from_numpy(rng.standard_normal((n, c)).astype(np.float32)).to(dtype)
     u2 = torch.from_numpy(rng.standard_normal((n, c)).astype(np.float32)).to(dtype)
     w = torch.from_numpy(rng.standard_normal((c, taps)).astype(np.float32)).to(dtype)
@@ -193,7 +193,7 @@ def test_causal_conv_across_portions(target, taps):
             pieces.append(u2[at2:at2 + k2])
             chunks.append((at2, k2))
             at2 += k2
-        y = sm.causal_conv(torch.cat(pieces).to(device), w.to(device), b.to(device), state, _sb(chunks, device, [2, 1][:len(chunks)]),
+        y = sm.causal_conv(torch.cat(pieces).to(device), w.t().contiguous().to(device), b.to(device), state, _sb(chunks, device, [2, 1][:len(chunks)]),
                            in_bias=ib.to(device))
         got.append(y[:k].cpu().numpy())
         at += k
@@ -201,12 +201,13 @@ def test_causal_conv_across_portions(target, taps):
 
 
 @pytest.mark.parametrize("target", TARGETS)
-def test_rglru_long_memory_across_portions(target):
+@pytest.mark.parametrize("blocks", [(3, 20), (2, 160)])
+def test_rglru_long_memory_across_portions(target, blocks):
     """Slow decays (lam very negative): the first tokens still weigh on the state hundreds of tokens
     later, so a state that is lost or reset between portions shows at the end."""
     device, dtype = _dev(target)
     rng = np.random.default_rng(5)
-    nb, bw, n = 3, 20, 300
+    (nb, bw), n = blocks, 300
     c = nb * bw
     f = lambda *s: rng.standard_normal(s).astype(np.float32)
     u, yraw = f(n, c), f(n, c)
