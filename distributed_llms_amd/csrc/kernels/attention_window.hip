@@ -10,7 +10,8 @@
 //                            threads laid out (value channel, key subgroup).  Decode rows, and prompt
 //                            chunks in float32.
 //   window_attn_tile_kernel  bf16 prompt chunks on MFMA (v_mfma_f32_16x16x32_bf16): one workgroup per
-//                            (64-query tile of a chunk, head), 4 waves x 16 queries, keys in tiles of 32
+//                            (64-query tile of a chunk, head), 4 waves x 16 queries, keys in tiles of 32 (the next tile's
+//                            global loads are in flight during the current tile's MFMAs)
 //                            staged through LDS (K rows permuted so that the S^T = K Q^T accumulator
 //                            hands each lane 8 consecutive keys, V transposed so that P.V reads 8 keys
 //                            of one value channel in one 16-byte load).  The softmax weights stay
@@ -174,11 +175,17 @@ static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
 
 
 // --------------------------------------------------------------------------- MFMA prompt kernel (bf16)
-constexpr int kTQ = 64;          // queries per workgroup (16 per wave)
+constexpr int kQT = 1;           // MFMA column tiles (16 queries) per wave: 1 keeps the kernel at <= 128 VGPRs
+                                 // (4 waves per SIMD, so one wave's softmax overlaps another's MFMAs); 2 halves the
+                                 // LDS reads per MFMA but measured slower at 1 wave per SIMD
+constexpr int kTQ = 64 * kQT;    // queries per workgroup: 4 waves x kQT column tiles
 constexpr int kTK = 32;          // keys per tile
 constexpr int kPad = 8;          // bf16 elements of row padding in LDS (16 bytes: rows start on different banks)
+constexpr float kLog2e = 1.4426950408889634f;
 
-// NQK: 32-wide K-dim steps of q.k (D <= 32 NQK); NDV: 16-wide tiles of value channels (Dv <= 16 NDV)
+// NQK: 32-wide K-dim steps of q.k (D <= 32 NQK); NDV: 16-wide tiles of value channels (Dv <= 16 NDV).
+// Every K / V^T fragment a wave reads from LDS feeds both of its query column tiles; the next key tile's
+// global loads are issued before the current tile's MFMAs and land in LDS after them.
 template <int NQK, int NDV>
 __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
@@ -186,6 +193,7 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int H, int G, int D, int Dv,
     int bs, int window, float scale) {
   constexpr int DP = 32 * NQK, KROW = DP + kPad, VROW = kTK + kPad;
+  constexpr int KPT = (kTK * (DP / 8) + 255) / 256, VPT = (16 * NDV * (kTK / 8) + 255) / 256;   // 16-byte pieces per thread
   __shared__ __attribute__((aligned(16))) bf16 ks[kTK * KROW];          // K tile, key j at row krow32(j)
   __shared__ __attribute__((aligned(16))) bf16 vs[16 * NDV * VROW];     // V^T tile [channel][key]
   const int b = seq0 + blockIdx.y, h = blockIdx.z;
@@ -196,113 +204,172 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   const int g = h / (H / G);
   const int start = positions[lo_t];                                   // position of the chunk's first token
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
-  // this lane's query (MFMA column): local index, position, validity
-  const int ql = q0 + wave * 16 + col;
-  const bool qok = ql < n;
-  const int qpos = start + min(ql, n - 1);
-  // Q fragments: B operand, lane (col, grp) holds q[query col][32 s + 8 grp .. + 7]
-  bf16x8 qf[NQK];
-  {
-    const bf16* qrow = q + ((size_t)(lo_t + min(ql, n - 1)) * H + h) * D;
+  // this lane's two queries (MFMA columns of the wave's two column tiles)
+  int ql[kQT], qpos[kQT];
+  bool qok[kQT];
+  bf16x8 qf[kQT][NQK];
+#pragma unroll
+  for (int c2 = 0; c2 < kQT; ++c2) {
+    ql[c2] = q0 + wave * 16 * kQT + c2 * 16 + col;
+    qok[c2] = ql[c2] < n;
+    qpos[c2] = start + min(ql[c2], n - 1);
+    const bf16* qrow = q + ((size_t)(lo_t + min(ql[c2], n - 1)) * H + h) * D;
 #pragma unroll
     for (int s2 = 0; s2 < NQK; ++s2) {
       const int d0 = 32 * s2 + 8 * grp;
       bf16x8 v;
-      if (d0 + 8 <= D) v = *reinterpret_cast<const bf16x8*>(qrow + d0);
-      else {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = d0 + j < D ? qrow[d0 + j] : (bf16)0.f;
-      }
-      qf[s2] = v;
+      for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
+      if (d0 + 8 <= D) v = *reinterpret_cast<const bf16x8*>(qrow + d0);
+      qf[c2][s2] = v;
     }
   }
-  // zero the K padding columns once (d in [D, DP)): the loads below never write them
+  // zero both tiles once: the K padding columns (d in [D, DP)) and the V^T rows of channels >= Dv are
+  // never written again
   for (int i = tid; i < kTK * KROW; i += 256) ks[i] = (bf16)0.f;
   for (int i = tid; i < 16 * NDV * VROW; i += 256) vs[i] = (bf16)0.f;
-  f32x4 acc[NDV];
+  f32x4 acc[kQT][NDV];
 #pragma unroll
-  for (int i = 0; i < NDV; ++i) acc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, l = 0.f;
+  for (int c2 = 0; c2 < kQT; ++c2)
+#pragma unroll
+    for (int i = 0; i < NDV; ++i) acc[c2][i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m[kQT], l[kQT];
+#pragma unroll
+  for (int c2 = 0; c2 < kQT; ++c2) m[c2] = -INFINITY, l[c2] = 0.f;
   const int last_pos = start + min(q0 + kTQ, n) - 1;                   // newest key any query of the tile sees
   const int first_pos = max(0, start + q0 - window + 1);               // oldest
-  // this wave's queries see keys in [wlo, whi]
-  const int whi = start + min(q0 + wave * 16 + 15, n - 1), wlo = max(0, start + q0 + wave * 16 - window + 1);
   const int d8 = D >> 3;
-  __syncthreads();
-  for (int k0 = first_pos & ~(kTK - 1); k0 <= last_pos; k0 += kTK) {
-    // ---- stage the tile: K rows (16-byte pieces), V transposed (element-wise)
-    for (int i = tid; i < kTK * d8; i += 256) {
-      const int j = i / d8, c = i - j * d8;
-      const int kp = min(k0 + j, last_pos);
-      const size_t row = ((size_t)bt[kp / bs] * G + g) * bs + (kp % bs);
-      *reinterpret_cast<bf16x8*>(ks + krow32(j) * KROW + 8 * c) =
-          *reinterpret_cast<const bf16x8*>(k_cache + row * D + 8 * c);
+  const float sc2 = scale * kLog2e;
+  bf16x8 kreg[KPT], vreg[VPT];
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int r = 0; r < KPT; ++r) {
+      const int i = tid + 256 * r;
+      if (i < kTK * d8) {
+        const int j = i / d8, c = i - j * d8;
+        const int kp = min(k0 + j, last_pos);
+        const size_t row = ((size_t)bt[kp / bs] * G + g) * bs + (kp % bs);
+        kreg[r] = *reinterpret_cast<const bf16x8*>(k_cache + row * D + 8 * c);
+      }
     }
-    for (int i = tid; i < Dv * (kTK / 8); i += 256) {
-      const int ch = i / (kTK / 8), c = i - ch * (kTK / 8);
-      const int kp = min(k0 + 8 * c, last_pos & ~7);       // 8 keys of one block (bs % 8 == 0)
-      const size_t at = (((size_t)bt[kp / bs] * G + g) * Dv + ch) * bs + (kp % bs);
-      *reinterpret_cast<bf16x8*>(vs + ch * VROW + 8 * c) = *reinterpret_cast<const bf16x8*>(v_cache + at);
+#pragma unroll
+    for (int r = 0; r < VPT; ++r) {
+      const int i = tid + 256 * r;
+      if (i < Dv * (kTK / 8)) {
+        const int ch = i / (kTK / 8), c = i - ch * (kTK / 8);
+        const int kp = min(k0 + 8 * c, last_pos & ~7);     // 8 keys of one block (bs % 8 == 0)
+        const size_t at = (((size_t)bt[kp / bs] * G + g) * Dv + ch) * bs + (kp % bs);
+        vreg[r] = *reinterpret_cast<const bf16x8*>(v_cache + at);
+      }
     }
+  };
+  auto stage = [&]() {
+#pragma unroll
+    for (int r = 0; r < KPT; ++r) {
+      const int i = tid + 256 * r;
+      if (i < kTK * d8) {
+        const int j = i / d8, c = i - j * d8;
+        *reinterpret_cast<bf16x8*>(ks + krow32(j) * KROW + 8 * c) = kreg[r];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < VPT; ++r) {
+      const int i = tid + 256 * r;
+      if (i < Dv * (kTK / 8)) {
+        const int ch = i / (kTK / 8), c = i - ch * (kTK / 8);
+        *reinterpret_cast<bf16x8*>(vs + ch * VROW + 8 * c) = vreg[r];
+      }
+    }
+  };
+  // keys the wave's queries see: [wlo, whi]
+  const int wq0 = q0 + wave * 16 * kQT;
+  const int whi = start + min(wq0 + 16 * kQT - 1, n - 1), wlo = max(0, start + wq0 - window + 1);
+  // a tile whose keys every query of the wave sees needs no mask: all keys <= the wave's first query's
+  // position and inside the window of its last one
+  const int full_hi = start + wq0, full_lo = whi - window + 1;
+  const bool wave_full = wq0 + 16 * kQT <= n;
+  const int kfirst = first_pos & ~(kTK - 1);
+  fetch(kfirst);
+  for (int k0 = kfirst; k0 <= last_pos; k0 += kTK) {
+    __syncthreads();                       // every wave is done with the previous tile
+    stage();
     __syncthreads();
+    if (k0 + kTK <= last_pos) fetch(k0 + kTK);
     if (k0 <= whi && k0 + kTK - 1 >= wlo) {
-      // ---- S^T = K Q^T: lane (col, grp) gets keys k0 + 8 grp + (0..7) of query col
-      f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+      // ---- S^T = K Q^T: lane (col, grp) gets keys k0 + 8 grp + (0..7) of its query in each column tile
+      f32x4 s0[kQT], s1[kQT];
+#pragma unroll
+      for (int c2 = 0; c2 < kQT; ++c2) s0[c2] = f32x4{0.f, 0.f, 0.f, 0.f}, s1[c2] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int s2 = 0; s2 < NQK; ++s2) {
         const bf16x8 ka = *reinterpret_cast<const bf16x8*>(ks + col * KROW + 32 * s2 + 8 * grp);
         const bf16x8 kb = *reinterpret_cast<const bf16x8*>(ks + (16 + col) * KROW + 32 * s2 + 8 * grp);
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[s2], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qf[s2], s1, 0, 0, 0);
-      }
-      float p[8];
-      float cm = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const int kp = k0 + 8 * grp + i;
-        const float sv = (i < 4 ? s0[i] : s1[i - 4]) * scale;
-        const bool ok = qok && kp <= qpos && qpos - kp < window;
-        p[i] = ok ? sv : -INFINITY;
-        cm = fmaxf(cm, p[i]);
+        for (int c2 = 0; c2 < kQT; ++c2) {
+          s0[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[c2][s2], s0[c2], 0, 0, 0);
+          s1[c2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qf[c2][s2], s1[c2], 0, 0, 0);
+        }
       }
-      cm = rows_max(cm);
-      const float m_new = fmaxf(m, cm);
-      const float m_use = m_new == -INFINITY ? 0.f : m_new;
-      const float alpha = m == -INFINITY ? 0.f : expf(m - m_new);
-      float ps = 0.f;
-      bf16x8 ph, pl;
+      const bool nomask = wave_full && k0 + kTK - 1 <= full_hi && k0 >= full_lo;    // wave-uniform
+      bf16x8 ph[kQT], pl[kQT];
+      float alpha[kQT];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float e = expf(p[i] - m_use);
-        ps += e;
-        ph[i] = (bf16)e;
-        pl[i] = (bf16)(e - (float)ph[i]);
+      for (int c2 = 0; c2 < kQT; ++c2) {
+        float p[8];
+        float cm = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const int kp = k0 + 8 * grp + i;
+          const float sv = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
+          const bool ok = nomask || (qok[c2] && kp <= qpos[c2] && qpos[c2] - kp < window);
+          p[i] = ok ? sv : -INFINITY;
+          cm = fmaxf(cm, p[i]);
+        }
+        cm = rows_max(cm);
+        const float m_new = fmaxf(m[c2], cm);
+        const float m_use = m_new == -INFINITY ? 0.f : m_new;
+        alpha[c2] = m[c2] == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m[c2] - m_new);
+        float ps = 0.f;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          const float e = __builtin_amdgcn_exp2f(p[i] - m_use);
+          ps += e;
+          ph[c2][i] = (bf16)e;
+          pl[c2][i] = (bf16)(e - (float)ph[c2][i]);
+        }
+        l[c2] = l[c2] * alpha[c2] + rows_sum(ps);
+        m[c2] = m_new;
       }
-      l = l * alpha + rows_sum(ps);
-      m = m_new;
 #pragma unroll
       for (int dt = 0; dt < NDV; ++dt) {
         if (16 * dt < Dv) {
           // A operand: V^T[channel 16 dt + col][keys 8 grp .. + 7]
           const bf16x8 va = *reinterpret_cast<const bf16x8*>(vs + (16 * dt + col) * VROW + 8 * grp);
-          f32x4 a = acc[dt] * alpha;
-          a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, ph, a, 0, 0, 0);
-          acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl, a, 0, 0, 0);
+#pragma unroll
+          for (int c2 = 0; c2 < kQT; ++c2) {
+            f32x4 a = acc[c2][dt] * alpha[c2];
+            a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, ph[c2], a, 0, 0, 0);
+            acc[c2][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl[c2], a, 0, 0, 0);
+          }
         }
       }
     }
-    __syncthreads();
   }
-  // O^T accumulator: lane (col, grp) holds channels 16 dt + 4 grp + (0..3) of query col
-  if (!qok) return;
-  const float inv = 1.0f / l;
-  bf16* orow = out + ((size_t)(lo_t + ql) * H + h) * Dv;
+  // O^T accumulator: lane (col, grp) holds channels 16 dt + 4 grp + (0..3) of its query
 #pragma unroll
-  for (int dt = 0; dt < NDV; ++dt) {
+  for (int c2 = 0; c2 < kQT; ++c2) {
+    if (!qok[c2]) continue;
+    const float inv = 1.0f / l[c2];
+    bf16* orow = out + ((size_t)(lo_t + ql[c2]) * H + h) * Dv;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int e = 16 * dt + 4 * grp + i;
-      if (e < Dv) orow[e] = (bf16)(acc[dt][i] * inv);
+    for (int dt = 0; dt < NDV; ++dt) {
+      const int e0 = 16 * dt + 4 * grp;
+      if (e0 + 4 <= Dv) {
+        bf16x4 o4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) o4[i] = (bf16)(acc[c2][dt][i] * inv);
+        *reinterpret_cast<bf16x4*>(orow + e0) = o4;
+      }
     }
   }
 }
@@ -317,7 +384,6 @@ static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
                      (const int32_t*)positions, seq0, H, G, D, Dv, bs, window, scale);
   DLLM_HIP_CHECK(hipGetLastError());
 }
-
 
 // --------------------------------------------------------------------------- MFMA decode kernel (bf16)
 // One workgroup per (one-token sequence, K/V head): the 16 MFMA columns are the query heads of the
@@ -362,29 +428,46 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   float m = -INFINITY, l = 0.f;
   // keys of this lane's A rows inside a tile: first half row col -> key 8 (col / 4) + col % 4, second half + 4
   const int jr = 8 * (col >> 2) + (col & 3);
-  for (int k0 = (lo & ~31) + 32 * wave; k0 <= pos; k0 += 32 * kDW) {
+  bf16x8 ka[NQK], kb[NQK];
+  auto load_k = [&](int k0) {
     const int j1 = min(k0 + jr, pos), j2 = min(k0 + jr + 4, pos);
     const bf16* r1 = k_cache + (((size_t)bt[j1 / bs] * G + g) * bs + j1 % bs) * D;
     const bf16* r2 = k_cache + (((size_t)bt[j2 / bs] * G + g) * bs + j2 % bs) * D;
-    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int s2 = 0; s2 < NQK; ++s2) {
       const int d0 = 32 * s2 + 8 * grp;
-      if (32 * s2 < D) {
-        bf16x8 ka, kb;
 #pragma unroll
-        for (int j = 0; j < 8; ++j) ka[j] = kb[j] = (bf16)0.f;
-        if (d0 + 8 <= D) {
-          ka = *reinterpret_cast<const bf16x8*>(r1 + d0);
-          kb = *reinterpret_cast<const bf16x8*>(r2 + d0);
-        }
-        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka, qf[s2], s0, 0, 0, 0);
-        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb, qf[s2], s1, 0, 0, 0);
+      for (int j = 0; j < 8; ++j) ka[s2][j] = kb[s2][j] = (bf16)0.f;
+      if (d0 + 8 <= D) {
+        ka[s2] = *reinterpret_cast<const bf16x8*>(r1 + d0);
+        kb[s2] = *reinterpret_cast<const bf16x8*>(r2 + d0);
       }
     }
-    // the V^T pieces of this lane: 8 keys from k0 + 8 grp (clamped to the last piece that exists)
+  };
+  const int kbeg = (lo & ~31) + 32 * wave;
+  if (kbeg <= pos) load_k(kbeg);
+  for (int k0 = kbeg; k0 <= pos; k0 += 32 * kDW) {
+    // this tile's V^T pieces (8 keys from k0 + 8 grp, clamped to the last piece that exists) go out first
     const int kp8 = min(k0 + 8 * grp, pos & ~7);
     const bf16* vbase = v_cache + ((size_t)bt[kp8 / bs] * G + g) * Dv * bs + kp8 % bs;
+    bf16x8 va[NDV];
+#pragma unroll
+    for (int dt = 0; dt < NDV; ++dt) {
+      const int ch = 16 * dt + col;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) va[dt][j] = (bf16)0.f;
+      if (ch < Dv) va[dt] = *reinterpret_cast<const bf16x8*>(vbase + (size_t)ch * bs);
+    }
+    f32x4 s0 = {0.f, 0.f, 0.f, 0.f}, s1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s2 = 0; s2 < NQK; ++s2) {
+      if (32 * s2 < D) {
+        s0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ka[s2], qf[s2], s0, 0, 0, 0);
+        s1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kb[s2], qf[s2], s1, 0, 0, 0);
+      }
+    }
+    // the wave's next tile's K rows are in flight during this tile's softmax and P.V
+    if (k0 + 32 * kDW <= pos) load_k(k0 + 32 * kDW);
     float p[8];
     float cm = -INFINITY;
 #pragma unroll
@@ -412,14 +495,9 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
 #pragma unroll
     for (int dt = 0; dt < NDV; ++dt) {
       if (16 * dt < Dv) {
-        const int ch = 16 * dt + col;
-        bf16x8 va;
-#pragma unroll
-        for (int j = 0; j < 8; ++j) va[j] = (bf16)0.f;
-        if (ch < Dv) va = *reinterpret_cast<const bf16x8*>(vbase + (size_t)ch * bs);
         f32x4 a = acc[dt] * alpha;
-        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, ph, a, 0, 0, 0);
-        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl, a, 0, 0, 0);
+        a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], ph, a, 0, 0, 0);
+        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va[dt], pl, a, 0, 0, 0);
       }
     }
   }

@@ -21,7 +21,10 @@ template <typename T> __device__ __forceinline__ void stf(T* p, float v) { *p = 
 // V consecutive elements <-> float registers: V = 8 moves 16 bytes of bf16 (32 of float) per lane and
 // needs the address aligned to 8 elements; V = 1 is the any-size form.
 template <int V> __device__ __forceinline__ void ldv(const bf16* p, float (&o)[V]) {
-  if constexpr (V == 8) {
+  if constexpr (V == 2) {
+    const bf16x2 v = *reinterpret_cast<const bf16x2*>(p);
+    o[0] = bf2f(v[0]), o[1] = bf2f(v[1]);
+  } else if constexpr (V == 8) {
     const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
 #pragma unroll
     for (int j = 0; j < 8; ++j) o[j] = bf2f(v[j]);
@@ -31,7 +34,10 @@ template <int V> __device__ __forceinline__ void ldv(const bf16* p, float (&o)[V
   }
 }
 template <int V> __device__ __forceinline__ void ldv(const float* p, float (&o)[V]) {
-  if constexpr (V == 8) {
+  if constexpr (V == 2) {
+    const f32x2 v = *reinterpret_cast<const f32x2*>(p);
+    o[0] = v[0], o[1] = v[1];
+  } else if constexpr (V == 8) {
     const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
 #pragma unroll
     for (int j = 0; j < 4; ++j) o[j] = a[j], o[4 + j] = b[j];
@@ -41,7 +47,11 @@ template <int V> __device__ __forceinline__ void ldv(const float* p, float (&o)[
   }
 }
 template <int V> __device__ __forceinline__ void stv(bf16* p, const float (&o)[V]) {
-  if constexpr (V == 8) {
+  if constexpr (V == 2) {
+    bf16x2 v;
+    v[0] = f2bf(o[0]), v[1] = f2bf(o[1]);
+    *reinterpret_cast<bf16x2*>(p) = v;
+  } else if constexpr (V == 8) {
     bf16x8 v;
 #pragma unroll
     for (int j = 0; j < 8; ++j) v[j] = f2bf(o[j]);
@@ -52,7 +62,9 @@ template <int V> __device__ __forceinline__ void stv(bf16* p, const float (&o)[V
   }
 }
 template <int V> __device__ __forceinline__ void stv(float* p, const float (&o)[V]) {
-  if constexpr (V == 8) {
+  if constexpr (V == 2) {
+    *reinterpret_cast<f32x2*>(p) = f32x2{o[0], o[1]};
+  } else if constexpr (V == 8) {
     *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
     *reinterpret_cast<f32x4*>(p + 4) = f32x4{o[4], o[5], o[6], o[7]};
   } else {
@@ -393,6 +405,80 @@ __global__ void __launch_bounds__(256) sm_rglru_gates_small_kernel(float* __rest
   }
 }
 
+// The same for blocks whose width is a multiple of 8: a lane loads 8 consecutive outputs of one input
+// row (16 bytes of bf16) and the workgroup's 8 lane groups take every 8th input row; their partial
+// sums meet in LDS.  256 outputs of block b per workgroup.
+template <typename T>
+__global__ void __launch_bounds__(256) sm_rglru_gates_small_vec_kernel(
+    float* __restrict__ a_out, float* __restrict__ g_out, const float* __restrict__ u, const void* __restrict__ ra_t_,
+    const void* __restrict__ ra_b_, const void* __restrict__ ri_t_, const void* __restrict__ ri_b_,
+    const void* __restrict__ lam_, int tokens, int nb, int bw, float scale) {
+  extern __shared__ float smem[];
+  float* ubs = smem;                                  // [GT][bw]
+  float* red = smem + GT * bw;                        // [8 groups][GT][256]
+  const int t0 = blockIdx.x * GT, b = blockIdx.y, C = nb * bw, o0 = blockIdx.z * 256;
+  const int nt = min(GT, tokens - t0);
+  const int tid = threadIdx.x, og = tid & 31, kg = tid >> 5;
+  for (int i = tid; i < GT * bw; i += 256) {
+    const int k = i / bw, c = i - k * bw;
+    ubs[i] = k < nt ? u[(size_t)(t0 + k) * C + b * bw + c] : 0.f;
+  }
+  __syncthreads();
+  const T* ra = (const T*)ra_t_ + (size_t)b * bw * bw;
+  const T* ri = (const T*)ri_t_ + (size_t)b * bw * bw;
+  const int ob = o0 + 8 * og;                         // this lane's 8 outputs
+  float ar[GT][8], ai[GT][8];
+#pragma unroll
+  for (int k = 0; k < GT; ++k)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) ar[k][j] = 0.f, ai[k][j] = 0.f;
+  if (ob < bw) {
+    for (int i = kg; i < bw; i += 8) {
+      float wr[8], wi[8];
+      ldv<8>(ra + (size_t)i * bw + ob, wr);
+      ldv<8>(ri + (size_t)i * bw + ob, wi);
+#pragma unroll
+      for (int k = 0; k < GT; ++k) {
+        const float x = ubs[k * bw + i];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) ar[k][j] = fmaf(wr[j], x, ar[k][j]), ai[k][j] = fmaf(wi[j], x, ai[k][j]);
+      }
+    }
+  }
+  // the 8 lane groups' partial sums meet in LDS, one gate after the other (the same 32 KiB)
+  float sr[GT], si[GT];
+#pragma unroll
+  for (int pass = 0; pass < 2; ++pass) {
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < GT; ++k)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) red[(kg * GT + k) * 256 + 8 * og + j] = pass ? ai[k][j] : ar[k][j];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < GT; ++k) {                    // this thread finishes (token k, output o0 + tid)
+      float sum = 0.f;
+#pragma unroll
+      for (int g8 = 0; g8 < 8; ++g8) sum += red[(g8 * GT + k) * 256 + tid];
+      if (pass) si[k] = sum; else sr[k] = sum;
+    }
+  }
+  const int o = o0 + tid;
+  if (o >= bw) return;
+  const int ch = b * bw + o;
+  const float sp = softplus_f(ldf((const T*)lam_ + ch));
+  const float rb = ldf((const T*)ra_b_ + ch), ib = ldf((const T*)ri_b_ + ch);
+#pragma unroll
+  for (int k = 0; k < GT; ++k) {
+    if (k < nt) {
+      const float av = expf(-scale * sigmoid_f(sr[k] + rb) * sp);
+      const size_t at = (size_t)(t0 + k) * C + ch;
+      a_out[at] = av;
+      g_out[at] = sqrtf(1.0f - av * av) * sigmoid_f(si[k] + ib) * ubs[k * bw + o];
+    }
+  }
+}
+
 // Many tokens (prompts): the two block-diagonal products on the float32 matrix cores
 // (v_mfma_f32_32x32x2_f32: true 32-bit operands and sums, which the gates of the recurrence require).
 // One workgroup per (64 tokens, block b, 128 outputs of the block): each wave owns 32 outputs and, for
@@ -479,6 +565,13 @@ void sm_rglru_gates(uintptr_t a, uintptr_t g, uintptr_t u, uintptr_t ra_t, uintp
   if (tokens <= 0) return;
   DLLM_HOST_CHECK(nb > 0 && bw > 0 && nb <= 65535 && (bw + 127) / 128 <= 65535, "rglru gate sizes");
   const size_t lds = (size_t)GT * bw * sizeof(float);
+  const size_t lds_vec = lds + (size_t)8 * GT * 256 * sizeof(float);
+  if (tokens <= 64 && bw % 8 == 0 && lds_vec <= 64 * 1024) {
+    SM_DISPATCH(f32, sm_rglru_gates_small_vec_kernel, dim3((tokens + GT - 1) / GT, nb, (bw + 255) / 256), dim3(256),
+                lds_vec, stream, (float*)a, (float*)g, (const float*)u, (const void*)ra_t, (const void*)ra_b,
+                (const void*)ri_t, (const void*)ri_b, (const void*)lam, tokens, nb, bw, scale);
+    return;
+  }
   if (tokens <= 64 && lds <= 48 * 1024) {
     SM_DISPATCH(f32, sm_rglru_gates_small_kernel, dim3((tokens + GT - 1) / GT, nb), dim3(256), lds, stream, (float*)a,
                 (float*)g, (const float*)u, (const void*)ra_t, (const void*)ra_b, (const void*)ri_t,
@@ -670,6 +763,93 @@ __global__ void __launch_bounds__(64) sm_attn_prep_kernel(
   }
 }
 
+// The same with even head sizes: a lane owns rotation pairs (channels 2e, 2e + 1), so the convolution
+// reads 2-element vectors, the rotation needs no exchange through LDS, and q / k leave as 2-element
+// stores.  Heads up to 512 wide (4 pairs per lane).
+constexpr int kPrepPairs = 4;
+
+template <typename T>
+__global__ void __launch_bounds__(256) sm_attn_prep_pair_kernel(
+    void* __restrict__ q_out_, const void* __restrict__ qkv_, const void* __restrict__ conv_w_,
+    const void* __restrict__ state_, const void* __restrict__ q_norm_, const void* __restrict__ k_norm_,
+    const float* __restrict__ freqs, int nrot, float mag, float eps, void* __restrict__ k_cache_,
+    void* __restrict__ v_cache_, const int32_t* __restrict__ slot_mapping, const int32_t* __restrict__ cu,
+    const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, const int32_t* __restrict__ slots,
+    int H, int G, int D, int Dv, int taps, int bs) {
+  const int t = blockIdx.x, head = blockIdx.y * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;   // a wave per head
+  if (head >= H + 2 * G) return;
+  const int C = H * D + G * (D + Dv);
+  const int b = tok_seq[t];
+  const int tl = t - cu[b], pos = positions[t];
+  const T* qkv = (const T*)qkv_;
+  const T* w = (const T*)conv_w_;
+  const T* st = (const T*)state_ + (size_t)slots[b] * (taps - 1) * C;
+  int c0, n, kind;                                   // kind 0 q, 1 k, 2 v
+  if (head < H) c0 = head * D, n = D, kind = 0;
+  else if (head < H + G) c0 = H * D + (head - H) * D, n = D, kind = 1;
+  else c0 = H * D + G * D + (head - H - G) * Dv, n = Dv, kind = 2;
+  float x[kPrepPairs][2];
+  float ss = 0.f;
+#pragma unroll
+  for (int r = 0; r < kPrepPairs; ++r) {
+    const int e = 2 * (lane + 64 * r);
+    x[r][0] = x[r][1] = 0.f;
+    if (e < n) {
+      const int c = c0 + e;
+      for (int j = 0; j < taps; ++j) {
+        const int d = taps - 1 - j;
+        if (d > pos) continue;
+        float xv[2], wv[2];
+        if (d <= tl) ldv<2>(qkv + (size_t)(t - d) * C + c, xv);
+        else ldv<2>(st + (size_t)(tl - d + taps - 1) * C + c, xv);
+        ldv<2>(w + (size_t)j * C + c, wv);
+        x[r][0] += wv[0] * xv[0];
+        x[r][1] += wv[1] * xv[1];
+      }
+      ss += x[r][0] * x[r][0] + x[r][1] * x[r][1];
+    }
+  }
+  if (kind == 2) {
+    const int slot = slot_mapping[t];
+    const int blk = slot / bs, off = slot - blk * bs;
+    T* dst = (T*)v_cache_ + ((size_t)blk * G + (head - H - G)) * Dv * bs + off;
+#pragma unroll
+    for (int r = 0; r < kPrepPairs; ++r) {
+      const int e = 2 * (lane + 64 * r);
+      if (e < n) stf(dst + (size_t)e * bs, x[r][0]), stf(dst + (size_t)(e + 1) * bs, x[r][1]);
+    }
+    return;
+  }
+  T* dst;
+  if (kind == 0) dst = (T*)q_out_ + ((size_t)t * H + head) * D;
+  else {
+    const int slot = slot_mapping[t];
+    const int blk = slot / bs, off = slot - blk * bs;
+    dst = (T*)k_cache_ + (((size_t)blk * G + (head - H)) * bs + off) * D;
+  }
+  ss = wave_sum(ss);
+  const float inv = 1.0f / sqrtf(ss / (float)n + eps);
+  const T* nw = (const T*)(kind == 0 ? q_norm_ : k_norm_);
+  const float fpos = (float)pos;
+#pragma unroll
+  for (int r = 0; r < kPrepPairs; ++r) {
+    const int i = lane + 64 * r, e = 2 * i;
+    if (e < n) {
+      float g2[2], o[2];
+      ldv<2>(nw + e, g2);
+      float x0 = x[r][0] * inv * g2[0], x1 = x[r][1] * inv * g2[1];
+      if (i < nrot) {
+        const float ang = fpos * freqs[i];
+        const float cs = cosf(ang) * mag, sn = sinf(ang) * mag;
+        const float r0 = x0 * cs - x1 * sn, r1 = x1 * cs + x0 * sn;
+        x0 = r0, x1 = r1;
+      }
+      o[0] = x0, o[1] = x1;
+      stv<2>(dst + e, o);
+    }
+  }
+}
+
 void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t state, uintptr_t q_norm,
                   uintptr_t k_norm, uintptr_t freqs, int nrot, float mag, float eps, uintptr_t k_cache,
                   uintptr_t v_cache, uintptr_t slot_mapping, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq,
@@ -681,6 +861,13 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
   DLLM_HOST_CHECK(H + 2 * G <= 65535, "attn_prep heads");
   const int C = H * D + G * (D + Dv);
   const size_t lds = (size_t)std::max(D, Dv) * sizeof(float);
+  if (D % 2 == 0 && Dv % 2 == 0 && std::max(D, Dv) <= 128 * kPrepPairs)
+    SM_DISPATCH(f32, sm_attn_prep_pair_kernel, dim3(tokens, (H + 2 * G + 3) / 4), dim3(256), 0, stream, (void*)q_out,
+                (const void*)qkv, (const void*)conv_w, (const void*)state, (const void*)q_norm, (const void*)k_norm,
+                (const float*)freqs, nrot, mag, eps, (void*)k_cache, (void*)v_cache, (const int32_t*)slot_mapping,
+                (const int32_t*)cu, (const int32_t*)positions, (const int32_t*)tok_seq, (const int32_t*)slots, H, G, D,
+                Dv, taps, bs);
+  else
   SM_DISPATCH(f32, sm_attn_prep_kernel, dim3(tokens, H + 2 * G), dim3(64), lds, stream, (void*)q_out, (const void*)qkv,
               (const void*)conv_w, (const void*)state, (const void*)q_norm, (const void*)k_norm, (const float*)freqs,
               nrot, mag, eps, (void*)k_cache, (void*)v_cache, (const int32_t*)slot_mapping, (const int32_t*)cu,

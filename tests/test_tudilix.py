@@ -54,7 +54,7 @@ def cfg_a():
 
 def cfg_b():
     """Degenerate sizes: one tap (a convolution that is a scale), one block, one K/V head per query
-    head, a window longer than any test prompt, no soft cap, residual_mult 1, odd widths."""
+    head, a window longer than any test prompt, no soft cap, residual_mult 1, odd widths and head sizes."""
     return {"architecture": "Tudilix", "vocab": 131, "width": 72, "residual_mult": 1.0, "logit_softcap": 0.0,
             "norm": {"eps": 1e-5},
             "layers": [
@@ -63,7 +63,7 @@ def cfg_b():
                 {"type": "attention", "mixer": {"conv": 1, "dim": 20, "vdim": 12, "heads": 3, "kv_heads": 3,
                                                 "mask": {"size": 4096}, "scale": 0.25, "rot": _rot(20)},
                  "mlp": {"kind": "dense", "ff": 88, "limit": 5.0}},
-                {"type": "attention", "mixer": {"conv": 5, "dim": 16, "vdim": 16, "heads": 2, "kv_heads": 1,
+                {"type": "attention", "mixer": {"conv": 5, "dim": 17, "vdim": 9, "heads": 2, "kv_heads": 1,
                                                 "mask": {"size": 3}, "scale": 0.5, "rot": _rot(8, base=500.0)},
                  "mlp": None},
             ]}
