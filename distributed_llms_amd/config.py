@@ -204,7 +204,8 @@ def _from_layer_list(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelCo
         num_heads=max([m["heads"] for m in attn] or [1]), num_kv_heads=max([m["kv_heads"] for m in attn] or [1]),
         head_dim=max([max(m["dim"], m["vdim"]) for m in attn] or [1]), max_position=1 << 30,
         norm_eps=float(cfg["norm"]["eps"]), bos_token_id=-1, eos_token_id=-1, layers=layers,
-        residual_mult=float(cfg.get("residual_mult", 1.0)), logit_softcap=float(cfg.get("logit_softcap", 0.0)))
+        residual_mult=float(1.0 if cfg.get("residual_mult") is None else cfg["residual_mult"]),
+        logit_softcap=float(cfg.get("logit_softcap") or 0.0))
 
 
 ModelConfig.from_layer_list = staticmethod(_from_layer_list)

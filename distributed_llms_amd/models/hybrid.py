@@ -287,7 +287,9 @@ class HybridStage:
                          self.cfg.norm_eps, kc if own else None, vc if own else None, meta.slot_mapping, sb,
                          m["heads"], m["kv_heads"], m["dim"], m["vdim"])
         nd = meta.num_decode if meta.is_prefill else meta.num_seqs
-        a = sm.window_attention(q, kc, vc, meta.block_tables, sb, m["mask"]["size"], m["scale"], num_decode=nd)
+        window = int((m.get("mask") or {}).get("size") or (1 << 30))          # no mask entry: plain causal attention
+        scale = float(m["scale"]) if m.get("scale") is not None else m["dim"] ** -0.5
+        a = sm.window_attention(q, kc, vc, meta.block_tables, sb, window, scale, num_decode=nd)
         return ops.linear(a.view(a.shape[0], -1), w["wo"])
 
     def _rglru(self, i: int, h: torch.Tensor, w, sb: sm.SeqBatch) -> torch.Tensor:

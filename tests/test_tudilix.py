@@ -55,11 +55,11 @@ def cfg_a():
 def cfg_b():
     """Degenerate sizes: one tap (a convolution that is a scale), one block, one K/V head per query
     head, a window longer than any test prompt, no soft cap, residual_mult 1, odd widths and head sizes."""
-    return {"architecture": "Tudilix", "vocab": 131, "width": 72, "residual_mult": 1.0, "logit_softcap": 0.0,
+    return {"architecture": "Tudilix", "vocab": 131, "width": 76, "residual_mult": 1.0, "logit_softcap": 0.0,
             "norm": {"eps": 1e-5},
             "layers": [
-                {"type": "rglru", "mixer": {"blocks": 1, "conv": 1, "width": 40},
-                 "mlp": {"kind": "dense", "ff": 56, "limit": 0.8}},
+                {"type": "rglru", "mixer": {"blocks": 1, "conv": 1, "width": 42},
+                 "mlp": {"kind": "dense", "ff": 54, "limit": 0.8}},
                 {"type": "attention", "mixer": {"conv": 1, "dim": 20, "vdim": 12, "heads": 3, "kv_heads": 3,
                                                 "mask": {"size": 4096}, "scale": 0.25, "rot": _rot(20)},
                  "mlp": {"kind": "dense", "ff": 88, "limit": 5.0}},
