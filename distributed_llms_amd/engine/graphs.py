@@ -16,7 +16,8 @@ import torch
 from ..models.stage import BatchMeta, ModelStage
 from .batch import HostBatch, next_pow2
 
-SCRATCH_SEQ_ID = -1      # owns block 0 in the BlockManager
+SCRATCH_SEQ_ID = -1      # owns block 0 (and state slot 0) in the BlockManager
+NROWS = 5                # per-row int32 inputs: ids, positions, slots, seq_lens, state slots
 _CAPTURE_LOCK = threading.Lock()   # one graph capture at a time per process
 
 
@@ -34,21 +35,26 @@ class DecodeGraphRunner:
         cfg = stage.cfg
         mb, dev = self.max_batch, self.dev
         # every int32 graph input lives in ONE device buffer laid out like the pinned staging
-        # buffer -- [ids | positions | slots | seq_lens] x max_batch, then the block table rows --
-        # so a step's inputs go up in a single H2D copy (the first 4 * max_batch + bb * max_blocks
-        # ints) instead of five
-        self.dev_in = torch.zeros(4 * mb + mb * max_blocks, dtype=torch.int32, device=dev)
+        # buffer -- [ids | positions | slots | seq_lens | state slots] x max_batch, then the block
+        # table rows -- so a step's inputs go up in a single H2D copy (the first
+        # 5 * max_batch + bb * max_blocks ints) instead of six
+        self.dev_in = torch.zeros(NROWS * mb + mb * max_blocks, dtype=torch.int32, device=dev)
         self.ids = self.dev_in[0:mb]
         self.positions = self.dev_in[mb:2 * mb]
         self.slots = self.dev_in[2 * mb:3 * mb]
         self.seq_lens = self.dev_in[3 * mb:4 * mb]
         self.seq_lens.fill_(1)
-        self.block_tables = self.dev_in[4 * mb:].view(mb, max_blocks)
+        self.state_slots = self.dev_in[4 * mb:5 * mb]
+        self.block_tables = self.dev_in[NROWS * mb:].view(mb, max_blocks)
+        # models with per-sequence state: a decode step is one token per sequence, so the token ->
+        # sequence map and the chunk offsets are constants
+        self.with_state = bool(getattr(cfg, "needs_state_slots", False))
+        self.row_ids = torch.arange(mb + 1, dtype=torch.int32, device=dev) if self.with_state else None
         self.hidden = None if stage.is_first else torch.zeros(mb, stage.in_width, dtype=stage.dtype, device=dev)
         max_splits = 64
         self.ws = (torch.empty(mb * cfg.num_heads * max_splits * cfg.head_dim, dtype=torch.float32, device=dev),
                    torch.empty(mb * cfg.num_heads * max_splits * 2, dtype=torch.float32, device=dev))
-        self.pinned = torch.empty(4 * mb + mb * max_blocks, dtype=torch.int32).pin_memory()
+        self.pinned = torch.empty(NROWS * mb + mb * max_blocks, dtype=torch.int32).pin_memory()
         self.pinned_np = self.pinned.numpy()
         self.graphs: Dict[Tuple[int, int], Tuple[torch.cuda.CUDAGraph, torch.Tensor]] = {}
         self.pool = None
@@ -64,9 +70,14 @@ class DecodeGraphRunner:
         return b <= self.max_batch and max_ctx <= self.max_blocks * self.block_size
 
     def _meta(self, bb: int, cb: int) -> BatchMeta:
-        return BatchMeta(is_prefill=False, positions=self.positions[:bb], slot_mapping=self.slots[:bb],
+        meta = BatchMeta(is_prefill=False, positions=self.positions[:bb], slot_mapping=self.slots[:bb],
                          block_tables=self.block_tables[:bb], seq_lens=self.seq_lens[:bb], max_q_len=1,
                          max_ctx=cb, num_seqs=bb, num_tokens=bb, attn_workspace=self.ws)
+        if self.with_state:
+            meta.state_slots = self.state_slots[:bb]
+            meta.tok_seq = self.row_ids[:bb]
+            meta.cu_seqlens_q = self.row_ids[:bb + 1]
+        return meta
 
     def _inp(self, bb: int) -> torch.Tensor:
         return self.ids[:bb] if self.stage.is_first else self.hidden[:bb]
@@ -76,6 +87,11 @@ class DecodeGraphRunner:
             return self._capture(bb, cb)
 
     def _capture(self, bb: int, cb: int):
+        # the warm-up forwards below really run: every row is made a scratch row first (block 0,
+        # state slot 0, position 0), so they cannot advance a live sequence's recurrent state or
+        # convolution tail; run() loads the step's inputs after the capture
+        self.dev_in.zero_()
+        self.seq_lens.fill_(1)
         meta = self._meta(bb, cb)
         # warm up outside capture (allocator, lazy module init)
         if self.capture_stream is None:
@@ -107,19 +123,21 @@ class DecodeGraphRunner:
         # instead of one torch op (~5-10 us of host time each) per field
         n, mb, w = bb, self.max_batch, self.max_blocks
         p = self.pinned_np
-        pv = p[: 4 * mb].reshape(4, mb)
+        pv = p[: NROWS * mb].reshape(NROWS, mb)
         pv[0, :b] = hb.ids
         pv[1, :b] = hb.positions
         pv[2, :b] = hb.slots
         pv[3, :b] = hb.seq_lens
+        pv[4, :b] = hb.state_slots if hb.state_slots is not None else 0
         if n > b:                                       # padded rows: scratch slot 0, one token
             pv[:3, b:n] = 0
             pv[3, b:n] = 1
-        bt = p[4 * mb: 4 * mb + n * w].reshape(n, w)
+            pv[4, b:n] = 0
+        bt = p[NROWS * mb: NROWS * mb + n * w].reshape(n, w)
         bt[:b, :mbk] = hb.block_tables
         bt[:b, mbk:] = 0
         bt[b:] = 0
-        cnt = 4 * mb + n * w
+        cnt = NROWS * mb + n * w
         self.dev_in[:cnt].copy_(self.pinned[:cnt], non_blocking=True)
         if self.copy_done is None:
             self.copy_done = torch.cuda.Event()
@@ -135,12 +153,12 @@ class DecodeGraphRunner:
         ``ids_dev``: device-resident input ids overriding ``hb.ids`` (lookahead decode)."""
         b = hb.num_seqs
         bb, cb = self.bucket(b, hb.max_ctx)
+        entry = self.graphs.get((bb, cb))
+        if entry is None:
+            entry = self.capture(bb, cb)       # clears the input buffers: before this step's inputs go up
         self.load_inputs(hb, bb, hidden)
         if ids_dev is not None:
             self.ids[:b].copy_(ids_dev, non_blocking=True)
-        entry = self.graphs.get((bb, cb))
-        if entry is None:
-            entry = self.capture(bb, cb)
         g, out = entry
         g.replay()
         return out[:b]

@@ -87,7 +87,7 @@ def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int 
         tmp: str = "/tmp/dllm_hybrid_bench", models=("tudilix", "llama")) -> dict:
     out = {"size": size, "batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
            "data": "synthetic (random-init weights, random token ids)"}
-    for key, cfg, graphs in (("tudilix", hybrid_config(size), False), ("llama", llama_config(size), True)):
+    for key, cfg, graphs in (("tudilix", hybrid_config(size), True), ("llama", llama_config(size), True)):
         if key not in models:
             continue
         p, d = _measure(cfg, batch, prompt_len, gen_len, reps, f"{tmp}/{key}", graphs)

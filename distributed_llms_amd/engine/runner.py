@@ -73,9 +73,7 @@ class StageRunner:
         self.max_blocks = -(-ecfg.max_seq_len // self.block_size)
         self._busy = None                 # [(start, end) events or host seconds] while metering
         self.graph_sets = []
-        # decode graphs replay fixed buffers of the attention-only step; steps of models with state
-        # slots launch eagerly
-        if ecfg.use_graphs and stage.device.type == "cuda" and not stage.cfg.needs_state_slots:
+        if ecfg.use_graphs and stage.device.type == "cuda":
             sizes = [b for b in ecfg.graph_batch_sizes if b <= ecfg.max_batch] or [ecfg.max_batch]
             if max(sizes) < ecfg.max_batch:
                 sizes.append(ecfg.max_batch)

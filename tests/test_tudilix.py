@@ -77,7 +77,7 @@ def _round(sd, dtype):
     return {k: torch.from_numpy(v).to(dtype).float() for k, v in sd.items()}
 
 
-def make_engine(cfg, sd, target, tmp_path, max_tokens=512, max_requests=4, block_size=32):
+def make_engine(cfg, sd, target, tmp_path, max_tokens=512, max_requests=4, block_size=32, graphs=False):
     device, dtype = target
     if device == "cuda" and not torch.cuda.is_available():
         pytest.skip("no GPU")
@@ -88,7 +88,7 @@ def make_engine(cfg, sd, target, tmp_path, max_tokens=512, max_requests=4, block
                         dtype="float32" if dtype == torch.float32 else "bfloat16", max_batch=max_requests,
                         max_seq_len=max_tokens + 1, kv_block_size=block_size,
                         num_kv_blocks=-(-max_tokens // block_size) + max_requests + 1,
-                        max_prefill_tokens=max_tokens, use_graphs=False)
+                        max_prefill_tokens=max_tokens, use_graphs=graphs, graph_batch_sizes=(1, 2, 4))
     return LLMEngine(ecfg, stage)
 
 
@@ -480,3 +480,27 @@ def test_window_attention_shapes(target, shape):
     qd = torch.stack([x[-1] for x in qs]).contiguous().to(device)
     o = sm.window_attention(qd, kcs.to(device), vcs.to(device), bt, rows, window, d ** -0.5)
     np.testing.assert_allclose(o.float().cpu().numpy(), np.stack([w[-1] for w in wants]), rtol=t, atol=t)
+
+
+@pytest.mark.parametrize("target", [t for t in TARGETS if "gpu" in t.id])
+def test_decode_graphs_replay_like_eager_steps(target, tmp_path):
+    """Decode steps through captured HIP graphs (batch buckets 1, 2 and 4, so rows are padded with
+    scratch rows): dozens of replays with prompt portions of other requests in between, every
+    position against the oracle -- the capture's warm-up runs must not have advanced any live
+    sequence's recurrent state, and a replay must read the step's own slots."""
+    cfg = cfg_a()
+    sd = _round(O.make_weights(cfg, seed=8), target[1])
+    eng = make_engine(cfg, sd, target, tmp_path, graphs=True)
+    assert eng.runner.graphs is not None
+    prompts = prompts_for(cfg, [80, 61, 47], seed=13)
+    sched = [[("r0", 30)], [("r1", 20), ("r2", 5)]]
+    sched += [[("r0", 1), ("r1", 1), ("r2", 1)]] * 12            # bucket 4 with one padded row
+    sched += [[("r0", 1)]] * 10 + [[("r1", 1), ("r2", 1)]] * 9   # buckets 1 and 2
+    sched += [[("r2", 21)], [("r0", 1), ("r1", 1)], [("r0", 27), ("r1", 19)]]
+    got = replay(eng, sched, prompts)
+    assert eng.runner.graphs.graphs, "no decode graph was captured"
+    for n, p in prompts.items():
+        want, _ = O.forward(cfg, sd, p)
+        assert rel_err(got[n], want) < tol(target), n
+    outs = eng.generate(list(prompts.values())[:2], SamplingParams(max_new_tokens=12, ignore_eos=True))
+    assert all(len(o) == 12 for o in outs)
