@@ -190,19 +190,28 @@ template <int NQK, int NDV>
 __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
-    const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int H, int G, int D, int Dv,
-    int bs, int window, float scale) {
+    const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int nseq, int nqt, int H, int G,
+    int D, int Dv, int bs, int window, float scale) {
   constexpr int DP = 32 * NQK, KROW = DP + kPad, VROW = kTK + kPad;
   constexpr int KPT = (kTK * (DP / 8) + 255) / 256, VPT = (16 * NDV * (kTK / 8) + 255) / 256;   // 16-byte pieces per thread
   __shared__ __attribute__((aligned(16))) bf16 ks[kTK * KROW];          // K tile, key j at row krow32(j)
   __shared__ __attribute__((aligned(16))) bf16 vs[16 * NDV * VROW];     // V^T tile [channel][key]
-  const int b = seq0 + blockIdx.y, h = blockIdx.z;
+  // Workgroups are dealt to the 8 XCDs round-robin by their linear id.  The id is decoded so that
+  // every tile that reads one (sequence, K/V head) pair -- all its query tiles and the heads of the
+  // group -- runs on the same XCD, whose L2 then serves the re-reads of that pair's keys and values;
+  // within a pair the longest query tiles (most keys, causal) start first.
+  const int R = H / G, per_pair = nqt * R, pairs = nseq * G;
+  const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
+  const int pair = (slot / per_pair) * 8 + xcd, rem = slot % per_pair;
+  if (pair >= pairs) return;
+  const int b = seq0 + pair / G, g = pair % G;
+  const int h = g * R + rem % R;
   const int lo_t = cu[b], n = cu[b + 1] - lo_t;
-  const int q0 = blockIdx.x * kTQ;                                     // first local query of the tile
+  const int q0 = (nqt - 1 - rem / R) * kTQ;                            // first local query of the tile
   if (q0 >= n) return;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, grp = lane >> 4;
-  const int g = h / (H / G);
   const int start = positions[lo_t];                                   // position of the chunk's first token
+  const int bsh = __ffs(bs) - 1;                                       // bs is a power of two here
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   // this lane's two queries (MFMA columns of the wave's two column tiles)
   int ql[kQT], qpos[kQT];
@@ -241,45 +250,48 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   const int d8 = D >> 3;
   const float sc2 = scale * kLog2e;
   bf16x8 kreg[KPT], vreg[VPT];
+  // this thread's 16-byte pieces of a tile: K piece r = (key kj[r], columns 8 kc[r] ..), V piece r =
+  // (channel vch[r], keys 8 vc[r] ..); the same for every tile
+  int kj[KPT], kc[KPT], vch[VPT], vc[VPT];
+#pragma unroll
+  for (int r = 0; r < KPT; ++r) {
+    const int i = tid + 256 * r;
+    kj[r] = i < kTK * d8 ? i / d8 : -1;
+    kc[r] = i - max(kj[r], 0) * d8;
+  }
+#pragma unroll
+  for (int r = 0; r < VPT; ++r) {
+    const int i = tid + 256 * r;
+    vch[r] = i < Dv * (kTK / 8) ? i / (kTK / 8) : -1;
+    vc[r] = i & (kTK / 8 - 1);
+  }
   auto fetch = [&](int k0) {
 #pragma unroll
     for (int r = 0; r < KPT; ++r) {
-      const int i = tid + 256 * r;
-      if (i < kTK * d8) {
-        const int j = i / d8, c = i - j * d8;
+      if (kj[r] >= 0) {
+        const int j = kj[r], c = kc[r];
         const int kp = min(k0 + j, last_pos);
-        const size_t row = ((size_t)bt[kp / bs] * G + g) * bs + (kp % bs);
+        const size_t row = ((size_t)bt[kp >> bsh] * G + g) * bs + (kp & (bs - 1));
         kreg[r] = *reinterpret_cast<const bf16x8*>(k_cache + row * D + 8 * c);
       }
     }
 #pragma unroll
     for (int r = 0; r < VPT; ++r) {
-      const int i = tid + 256 * r;
-      if (i < Dv * (kTK / 8)) {
-        const int ch = i / (kTK / 8), c = i - ch * (kTK / 8);
+      if (vch[r] >= 0) {
+        const int ch = vch[r], c = vc[r];
         const int kp = min(k0 + 8 * c, last_pos & ~7);     // 8 keys of one block (bs % 8 == 0)
-        const size_t at = (((size_t)bt[kp / bs] * G + g) * Dv + ch) * bs + (kp % bs);
+        const size_t at = (((size_t)bt[kp >> bsh] * G + g) * Dv + ch) * bs + (kp & (bs - 1));
         vreg[r] = *reinterpret_cast<const bf16x8*>(v_cache + at);
       }
     }
   };
   auto stage = [&]() {
 #pragma unroll
-    for (int r = 0; r < KPT; ++r) {
-      const int i = tid + 256 * r;
-      if (i < kTK * d8) {
-        const int j = i / d8, c = i - j * d8;
-        *reinterpret_cast<bf16x8*>(ks + krow32(j) * KROW + 8 * c) = kreg[r];
-      }
-    }
+    for (int r = 0; r < KPT; ++r)
+      if (kj[r] >= 0) *reinterpret_cast<bf16x8*>(ks + krow32(kj[r]) * KROW + 8 * kc[r]) = kreg[r];
 #pragma unroll
-    for (int r = 0; r < VPT; ++r) {
-      const int i = tid + 256 * r;
-      if (i < Dv * (kTK / 8)) {
-        const int ch = i / (kTK / 8), c = i - ch * (kTK / 8);
-        *reinterpret_cast<bf16x8*>(vs + ch * VROW + 8 * c) = vreg[r];
-      }
-    }
+    for (int r = 0; r < VPT; ++r)
+      if (vch[r] >= 0) *reinterpret_cast<bf16x8*>(vs + vch[r] * VROW + 8 * vc[r]) = vreg[r];
   };
   // keys the wave's queries see: [wlo, whi]
   const int wq0 = q0 + wave * 16 * kQT;
@@ -317,13 +329,21 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
       for (int c2 = 0; c2 < kQT; ++c2) {
         float p[8];
         float cm = -INFINITY;
+        if (nomask) {                                      // wave-uniform: no per-element mask work
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-          const int kp = k0 + 8 * grp + i;
-          const float sv = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
-          const bool ok = nomask || (qok[c2] && kp <= qpos[c2] && qpos[c2] - kp < window);
-          p[i] = ok ? sv : -INFINITY;
-          cm = fmaxf(cm, p[i]);
+          for (int i = 0; i < 8; ++i) {
+            p[i] = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
+            cm = fmaxf(cm, p[i]);
+          }
+        } else {
+#pragma unroll
+          for (int i = 0; i < 8; ++i) {
+            const int kp = k0 + 8 * grp + i;
+            const float sv = (i < 4 ? s0[c2][i] : s1[c2][i - 4]) * sc2;
+            const bool ok = qok[c2] && kp <= qpos[c2] && qpos[c2] - kp < window;
+            p[i] = ok ? sv : -INFINITY;
+            cm = fmaxf(cm, p[i]);
+          }
         }
         cm = rows_max(cm);
         const float m_new = fmaxf(m[c2], cm);
@@ -340,6 +360,10 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
         l[c2] = l[c2] * alpha[c2] + rows_sum(ps);
         m[c2] = m_new;
       }
+      bool diff = false;
+#pragma unroll
+      for (int c2 = 0; c2 < kQT; ++c2) diff = diff || alpha[c2] != 1.0f;
+      const bool rescale = __any(diff);
 #pragma unroll
       for (int dt = 0; dt < NDV; ++dt) {
         if (16 * dt < Dv) {
@@ -347,7 +371,8 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
           const bf16x8 va = *reinterpret_cast<const bf16x8*>(vs + (16 * dt + col) * VROW + 8 * grp);
 #pragma unroll
           for (int c2 = 0; c2 < kQT; ++c2) {
-            f32x4 a = acc[c2][dt] * alpha[c2];
+            f32x4 a = acc[c2][dt];
+            if (rescale) a *= alpha[c2];                   // wave-uniform: skipped once every row's maximum has settled
             a = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, ph[c2], a, 0, 0, 0);
             acc[c2][dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(va, pl[c2], a, 0, 0, 0);
           }
@@ -378,10 +403,13 @@ template <int NQK, int NDV>
 static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t cu, uintptr_t positions, int seq0, int nseq, int max_q_len, int H,
                         int G, int D, int Dv, int bs, int window, float scale, uintptr_t stream) {
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV>), dim3((max_q_len + kTQ - 1) / kTQ, nseq, H),
+  const int nqt = (max_q_len + kTQ - 1) / kTQ;
+  const long per_xcd = (long)((nseq * G + 7) / 8) * nqt * (H / G);      // workgroups of one XCD
+  DLLM_HOST_CHECK(per_xcd * 8 < (1L << 31), "window attention grid");
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV>), dim3((unsigned)(per_xcd * 8)),
                      dim3(256), 0, (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
                      (const bf16*)v_cache, (const int32_t*)block_tables, max_blocks, (const int32_t*)cu,
-                     (const int32_t*)positions, seq0, H, G, D, Dv, bs, window, scale);
+                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, scale);
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
@@ -408,6 +436,7 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, grp = lane >> 4;
   const int pos = positions[t], b = tok_seq[t];
   const int lo = max(0, pos - window + 1);
+  const int bsh = __ffs(bs) - 1;                     // bs is a power of two here
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   bf16x8 qf[NQK];
   {
@@ -431,8 +460,8 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   bf16x8 ka[NQK], kb[NQK];
   auto load_k = [&](int k0) {
     const int j1 = min(k0 + jr, pos), j2 = min(k0 + jr + 4, pos);
-    const bf16* r1 = k_cache + (((size_t)bt[j1 / bs] * G + g) * bs + j1 % bs) * D;
-    const bf16* r2 = k_cache + (((size_t)bt[j2 / bs] * G + g) * bs + j2 % bs) * D;
+    const bf16* r1 = k_cache + (((size_t)bt[j1 >> bsh] * G + g) * bs + (j1 & (bs - 1))) * D;
+    const bf16* r2 = k_cache + (((size_t)bt[j2 >> bsh] * G + g) * bs + (j2 & (bs - 1))) * D;
 #pragma unroll
     for (int s2 = 0; s2 < NQK; ++s2) {
       const int d0 = 32 * s2 + 8 * grp;
@@ -449,7 +478,7 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   for (int k0 = kbeg; k0 <= pos; k0 += 32 * kDW) {
     // this tile's V^T pieces (8 keys from k0 + 8 grp, clamped to the last piece that exists) go out first
     const int kp8 = min(k0 + 8 * grp, pos & ~7);
-    const bf16* vbase = v_cache + ((size_t)bt[kp8 / bs] * G + g) * Dv * bs + kp8 % bs;
+    const bf16* vbase = v_cache + ((size_t)bt[kp8 >> bsh] * G + g) * Dv * bs + (kp8 & (bs - 1));
     bf16x8 va[NDV];
 #pragma unroll
     for (int dt = 0; dt < NDV; ++dt) {
@@ -538,7 +567,8 @@ static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr
 // bf16 with 16-byte rows and pieces goes to the matrix cores; float32 (the exact path), odd head sizes
 // and heads wider than 256 take the row kernel
 static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs) {
-  return !f32 && D % 8 == 0 && Dv % 8 == 0 && bs % 8 == 0 && D <= 256 && Dv <= 256 && G > 0 && H % G == 0;
+  return !f32 && D % 8 == 0 && Dv % 8 == 0 && bs % 8 == 0 && (bs & (bs - 1)) == 0 && D <= 256 && Dv <= 256 && G > 0 &&
+         H % G == 0;
 }
 
 // Decode rows: tokens [0, rows) are one-token sequences.
