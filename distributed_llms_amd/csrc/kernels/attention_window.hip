@@ -15,8 +15,8 @@
 //                            staged through LDS (K rows permuted so that the S^T = K Q^T accumulator
 //                            hands each lane 8 consecutive keys, V transposed so that P.V reads 8 keys
 //                            of one value channel in one 16-byte load).  The softmax weights stay
-//                            float32: P is fed to the matrix cores as a bf16 pair (high part + the
-//                            rounding remainder), two MFMAs per tile, so P.V carries 16 significand bits.
+//                            float32: P is fed to the matrix cores as a bf16 pair (upper half + the
+//                            remainder), two MFMAs per tile, so P.V carries 16 significand bits.
 #include <math.h>
 
 #include "common.h"
@@ -173,6 +173,24 @@ static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
+
+
+// Softmax weights for the matrix cores without giving up their float32 value: e = hi + lo with hi the
+// upper 16 bits of e (a bf16 by truncation), lo = e - hi (exact in float32) cut to bf16 the same way;
+// hi + lo carries 16 significand bits of e.  Two values are packed into a dword with one byte permute.
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void split_pack(const float (&e)[8], bf16x8& ph, bf16x8& pl) {
+  u32x4 h, l;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t a = __float_as_uint(e[2 * i]), b = __float_as_uint(e[2 * i + 1]);
+    const float la = e[2 * i] - __uint_as_float(a & 0xffff0000u), lb = e[2 * i + 1] - __uint_as_float(b & 0xffff0000u);
+    h[i] = __builtin_amdgcn_perm(b, a, 0x07060302u);
+    l[i] = __builtin_amdgcn_perm(__float_as_uint(lb), __float_as_uint(la), 0x07060302u);
+  }
+  ph = __builtin_bit_cast(bf16x8, h);
+  pl = __builtin_bit_cast(bf16x8, l);
+}
 
 // --------------------------------------------------------------------------- MFMA prompt kernel (bf16)
 constexpr int kQT = 1;           // MFMA column tiles (16 queries) per wave: 1 keeps the kernel at <= 128 VGPRs
@@ -352,11 +370,10 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
         float ps = 0.f;
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-          const float e = __builtin_amdgcn_exp2f(p[i] - m_use);
-          ps += e;
-          ph[c2][i] = (bf16)e;
-          pl[c2][i] = (bf16)(e - (float)ph[c2][i]);
+          p[i] = __builtin_amdgcn_exp2f(p[i] - m_use);
+          ps += p[i];
         }
+        split_pack(p, ph[c2], pl[c2]);
         l[c2] = l[c2] * alpha[c2] + rows_sum(ps);
         m[c2] = m_new;
       }
@@ -514,11 +531,10 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
     bf16x8 ph, pl;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      const float e = expf(p[i] - m_use);
-      ps += e;
-      ph[i] = (bf16)e;
-      pl[i] = (bf16)(e - (float)ph[i]);
+      p[i] = expf(p[i] - m_use);
+      ps += p[i];
     }
+    split_pack(p, ph, pl);
     l = l * alpha + rows_sum(ps);
     m = m_new;
 #pragma unroll

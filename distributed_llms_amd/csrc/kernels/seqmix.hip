@@ -516,26 +516,40 @@ __global__ void __launch_bounds__(256) sm_rglru_gates_kernel(float* __restrict__
       ub[r][k] = (t0 + r < tokens && k < kn) ? u[(size_t)(t0 + r) * C + b * bw + kc + k] : 0.f;
     }
     __syncthreads();
-    for (int ks0 = 0; 2 * ks0 < kn; ks0 += kGU) {
-      float br[kGU], bi[kGU], a0[kGU], a1[kGU];
+    // groups of kGU k-steps: the next group's weights and u values are loaded before the current
+    // group's 4 kGU MFMAs issue, so their latency hides behind 64-cycle matrix instructions
+    float br[2][kGU], bi[2][kGU], a0[2][kGU], a1[2][kGU];
+    auto load_group = [&](int ks0, int buf) {
 #pragma unroll
       for (int j = 0; j < kGU; ++j) {
         const int k = 2 * (ks0 + j) + half;                  // inside the chunk
         const bool ok = k < kn && o < bw;
         const size_t at = (size_t)(kc + min(k, kn - 1)) * bw + oc;
         const float wr = ldf(ra + at), wi = ldf(ri + at);
-        br[j] = ok ? wr : 0.f;
-        bi[j] = ok ? wi : 0.f;
+        br[buf][j] = ok ? wr : 0.f;
+        bi[buf][j] = ok ? wi : 0.f;
         const int kk = min(k, kGK - 1);
-        a0[j] = k < kn ? ub[n][kk] : 0.f;
-        a1[j] = k < kn ? ub[32 + n][kk] : 0.f;
+        a0[buf][j] = k < kn ? ub[n][kk] : 0.f;
+        a1[buf][j] = k < kn ? ub[32 + n][kk] : 0.f;
       }
+    };
+    auto mma_group = [&](int buf) {
 #pragma unroll
       for (int j = 0; j < kGU; ++j) {
-        cr0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[j], br[j], cr0, 0, 0, 0);
-        ci0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[j], bi[j], ci0, 0, 0, 0);
-        cr1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], br[j], cr1, 0, 0, 0);
-        ci1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[j], bi[j], ci1, 0, 0, 0);
+        cr0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[buf][j], br[buf][j], cr0, 0, 0, 0);
+        ci0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a0[buf][j], bi[buf][j], ci0, 0, 0, 0);
+        cr1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[buf][j], br[buf][j], cr1, 0, 0, 0);
+        ci1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a1[buf][j], bi[buf][j], ci1, 0, 0, 0);
+      }
+    };
+    load_group(0, 0);
+    for (int ks0 = 0; 2 * ks0 < kn; ks0 += 2 * kGU) {
+      const bool more1 = 2 * (ks0 + kGU) < kn, more2 = 2 * (ks0 + 2 * kGU) < kn;
+      if (more1) load_group(ks0 + kGU, 1);
+      mma_group(0);
+      if (more1) {
+        if (more2) load_group(ks0 + 2 * kGU, 0);
+        mma_group(1);
       }
     }
   }
