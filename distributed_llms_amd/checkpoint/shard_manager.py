@@ -233,7 +233,11 @@ def write_synthetic_checkpoint(preset: str, out_dir: str, seed: int = 0, dtype=t
     from ..config import get_model_config
     cfg = get_model_config(preset)
     os.makedirs(out_dir, exist_ok=True)
-    sd = W.synth_hf_state_dict(cfg, seed=seed, dtype=dtype)
+    if cfg.is_layer_list:
+        from ..models.hybrid import synth_state_dict
+        sd = synth_state_dict(cfg, seed=seed, dtype=dtype)
+    else:
+        sd = W.synth_hf_state_dict(cfg, seed=seed, dtype=dtype)
     with open(os.path.join(out_dir, "config.json"), "w") as f:
         json.dump(cfg.to_hf_config(), f, indent=1)
     if safetensors:

@@ -367,6 +367,8 @@ class EngineConfig:
         cfg = get_model_config(self.model if self.shard_dir is None else self.shard_dir)
         if self.num_workers > cfg.num_layers:
             raise ValueError(f"{self.num_workers} stages > {cfg.num_layers} layers")
+        if cfg.is_layer_list and self.num_workers > 1:
+            raise ValueError("a layer-list model runs as one stage: num_workers must be 1")
 
     def model_config(self) -> ModelConfig:
         return get_model_config(self.shard_dir or self.model)

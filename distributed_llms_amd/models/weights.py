@@ -197,18 +197,19 @@ def hf_head_names(cfg: ModelConfig) -> Dict[str, str]:
     return d
 
 
-_LAYER_RE = re.compile(r"(?:^|\.)(?:layers|h|blocks|layer)\.(\d+)\.")
+_LAYER_RE = re.compile(r"(?:^|\.)(?:layers|h|blocks|layer)\.(\d+)\.|^l(\d+)\.")
 
 
 def layer_of(key: str) -> Optional[int]:
     """Block index of an HF parameter name (``model.layers.N.``, ``transformer.h.N.``,
-    ``model.decoder.layers.N.``), or None for embeddings / final norm / head."""
+    ``model.decoder.layers.N.``; ``lN.`` of layer-list checkpoints), or None for embeddings / final
+    norm / head."""
     m = _LAYER_RE.search(key)
-    return int(m.group(1)) if m else None
+    return int(m.group(1) or m.group(2)) if m else None
 
 
 def is_embed_key(key: str) -> bool:
-    return any(s in key for s in ("embed_tokens", "wte", "wpe", "embed_positions"))
+    return key == "embed" or any(s in key for s in ("embed_tokens", "wte", "wpe", "embed_positions"))
 
 
 def synth_block(cfg: ModelConfig, layer: int, seed: int, dtype, device) -> Dict[str, torch.Tensor]:

@@ -76,13 +76,16 @@ def test_two_worker_pipeline_matches_single_process(cluster, model):
     assert {w["remote"]["role"] for w in st["workers"].values()} == {"driver", "follower"}
 
 
-def test_single_worker_engine(cluster):
+@pytest.mark.parametrize("model", ["synthetic:tiny-llama", "synthetic:tiny-tudilix"])
+def test_single_worker_engine(cluster, model):
+    """One worker owning every layer; tiny-tudilix: the layer-list hybrid model (state slots, its own
+    stage class) through the same master / worker command line."""
     make, _ = cluster
-    m = make("synthetic:tiny-llama", 1)
+    m = make(model, 1)
     m.assign_shards()
     m.distribute_shards(timeout=300)
     res = m.generate(PROMPTS, max_new_tokens=5, ignore_eos=True, timeout=120)
-    ref = LLMEngine(_cfg("synthetic:tiny-llama")).generate(PROMPTS, SamplingParams(max_new_tokens=5, ignore_eos=True))
+    ref = LLMEngine(_cfg(model)).generate(PROMPTS, SamplingParams(max_new_tokens=5, ignore_eos=True))
     assert [r["tokens"] for r in res] == ref
     chunks = list(m.stream(PROMPTS[1], max_new_tokens=5, ignore_eos=True, timeout=120))
     assert sum(chunks, []) == ref[1] and len(chunks) >= 2
@@ -130,19 +133,20 @@ def test_worker_failure_eviction_and_recovery(cluster):
     assert [r["tokens"] for r in res] == [r[:4] for r in ref[:2]]
 
 
-def test_checkpoint_shards_distributed_by_path(cluster, tmp_path):
+@pytest.mark.parametrize("preset,workers", [("tiny-gpt2", 2), ("tiny-tudilix", 1)])
+def test_checkpoint_shards_distributed_by_path(cluster, tmp_path, preset, workers):
     from distributed_llms_amd.checkpoint.shard_manager import write_synthetic_checkpoint
-    d = write_synthetic_checkpoint("tiny-gpt2", str(tmp_path / "ckpt"), seed=7)
+    d = write_synthetic_checkpoint(preset, str(tmp_path / "ckpt"), seed=7)
     make, _ = cluster
-    m = make(d, 2)
+    m = make(d, workers)
     m.assign_shards()
     m.distribute_shards(timeout=300)
     res = m.generate(PROMPTS, max_new_tokens=5, ignore_eos=True, timeout=120)
     from distributed_llms_amd.checkpoint.shard_manager import iter_checkpoint
-    from distributed_llms_amd.models.stage import ModelStage
+    from distributed_llms_amd.models import make_stage
     from distributed_llms_amd.config import get_model_config
     cfg = get_model_config(d)
-    st = ModelStage(cfg, 0, cfg.num_layers, "cpu", __import__("torch").float32).load_hf_state(dict(iter_checkpoint(d)))
+    st = make_stage(cfg, 0, cfg.num_layers, "cpu", __import__("torch").float32).load_hf_state(dict(iter_checkpoint(d)))
     ref = LLMEngine(_cfg(d), st).generate(PROMPTS, SamplingParams(max_new_tokens=5, ignore_eos=True))
     assert [r["tokens"] for r in res] == ref
 
