@@ -83,7 +83,7 @@ void sm_rglru_gates(uintptr_t a, uintptr_t g, uintptr_t u, uintptr_t ra_t, uintp
                     uintptr_t stream);
 void sm_rglru_scan(uintptr_t out, uintptr_t a, uintptr_t g, uintptr_t y_raw, long y_stride, uintptr_t y_bias,
                    uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t slots, int seqs, int C, int max_q_len,
-                   int f32, uintptr_t stream);
+                   uintptr_t ab, int f32, uintptr_t stream);
 void sm_clipped_glu(uintptr_t out, uintptr_t gu, uintptr_t bias, int tokens, int F, float limit, float alpha, int f32,
                     uintptr_t stream);
 void sm_softcap(uintptr_t out, uintptr_t x, long n, float cap, int f32, uintptr_t stream);

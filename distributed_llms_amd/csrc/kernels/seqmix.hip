@@ -646,11 +646,110 @@ __global__ void __launch_bounds__(64) sm_rglru_scan_kernel(void* __restrict__ ou
   *sp = s;
 }
 
+// Long chunks of few sequences: the recurrence S_t = a_t S_(t-1) + g_t is affine in S, so a chunk cut
+// into segments of kSeg tokens is scanned in two launches.  The first reduces every segment to its
+// composition (A = prod a_t, B = the segment scanned from zero); the second gives every (sequence,
+// segment) its start state -- the slot's state folded through the earlier segments' (A, B) -- and scans
+// the segment with outputs.  sequences x segments x channels / 64 waves instead of sequences x channels / 64.
+constexpr int kSeg = 128;
+
+__global__ void __launch_bounds__(64) sm_rglru_seg_reduce_kernel(float* __restrict__ ab, float* __restrict__ s0,
+                                                                 const float* __restrict__ a,
+                                                                 const float* __restrict__ g,
+                                                                 const float* __restrict__ state,
+                                                                 const int32_t* __restrict__ cu,
+                                                                 const int32_t* __restrict__ positions,
+                                                                 const int32_t* __restrict__ slots, int C, int nseg) {
+  const int b = blockIdx.y, sg = blockIdx.z;
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  const int lo = cu[b] + sg * kSeg, hi = min(cu[b + 1], lo + kSeg);
+  if (c >= C || lo >= hi) return;
+  // the sequence's state before this step, copied where the second launch reads it: that launch's last
+  // segment overwrites the slot while other segments may not have started yet
+  if (sg == 0) s0[(size_t)b * C + c] = positions[lo] > 0 ? state[(size_t)slots[b] * C + c] : 0.f;
+  float A = 1.f, B = 0.f;
+  int t = lo;
+  for (; t + 8 <= hi; t += 8) {
+    float av[8], gv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) av[j] = a[(size_t)(t + j) * C + c], gv[j] = g[(size_t)(t + j) * C + c];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) A *= av[j], B = fmaf(av[j], B, gv[j]);
+  }
+  for (; t < hi; ++t) {
+    const float av = a[(size_t)t * C + c];
+    A *= av, B = fmaf(av, B, g[(size_t)t * C + c]);
+  }
+  float* o = ab + (((size_t)b * nseg + sg) * 2) * C + c;
+  o[0] = A;
+  o[C] = B;
+}
+
+template <typename T>
+__global__ void __launch_bounds__(64) sm_rglru_seg_scan_kernel(void* __restrict__ out_, const float* __restrict__ a,
+                                                               const float* __restrict__ g,
+                                                               const void* __restrict__ y_raw_, long y_stride,
+                                                               const void* __restrict__ y_bias_,
+                                                               float* __restrict__ state, const float* __restrict__ ab,
+                                                               const float* __restrict__ s0,
+                                                               const int32_t* __restrict__ cu,
+                                                               const int32_t* __restrict__ slots, int C, int nseg) {
+  const int b = blockIdx.y, sg = blockIdx.z;
+  const int c = blockIdx.x * 64 + threadIdx.x;
+  const int first = cu[b], end = cu[b + 1];
+  const int lo = first + sg * kSeg, hi = min(end, lo + kSeg);
+  if (c >= C || lo >= hi) return;
+  const T* y_raw = (const T*)y_raw_;
+  T* out = (T*)out_;
+  float s = s0[(size_t)b * C + c];
+  for (int j = 0; j < sg; ++j) {                          // the earlier segments, composed
+    const float* p = ab + (((size_t)b * nseg + j) * 2) * C + c;
+    s = fmaf(p[0], s, p[C]);
+  }
+  const float yb = ldf((const T*)y_bias_ + c);
+  int t = lo;
+  for (; t + 8 <= hi; t += 8) {
+    float av[8], gv[8], yv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const size_t i = (size_t)(t + j) * C + c;
+      av[j] = a[i];
+      gv[j] = g[i];
+      yv[j] = ldf(y_raw + (size_t)(t + j) * y_stride + c);
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      s = fmaf(av[j], s, gv[j]);
+      stf(out + (size_t)(t + j) * C + c, s * gelu_tanh_f(yv[j] + yb));
+    }
+  }
+  for (; t < hi; ++t) {
+    const size_t i = (size_t)t * C + c;
+    s = fmaf(a[i], s, g[i]);
+    stf(out + i, s * gelu_tanh_f(ldf(y_raw + (size_t)t * y_stride + c) + yb));
+  }
+  if (hi == end) state[(size_t)slots[b] * C + c] = s;     // the sequence's last segment leaves the new state
+}
+
+// ab: workspace of seqs x (ceil(max_q_len / kSeg) x 2 + 1) x C floats (0: always the one-launch scan)
 void sm_rglru_scan(uintptr_t out, uintptr_t a, uintptr_t g, uintptr_t y_raw, long y_stride, uintptr_t y_bias,
                    uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t slots, int seqs, int C, int max_q_len,
-                   int f32, uintptr_t stream) {
+                   uintptr_t ab, int f32, uintptr_t stream) {
   if (seqs <= 0) return;
   DLLM_HOST_CHECK(C > 0 && y_stride >= C && seqs <= 65535, "rglru scan sizes");
+  const int nseg = (max_q_len + kSeg - 1) / kSeg;
+  if (ab && nseg > 1 && nseg <= 65535) {
+    const dim3 grid((C + 63) / 64, seqs, nseg);
+    float* s0 = (float*)ab + (size_t)seqs * nseg * 2 * C;
+    hipLaunchKernelGGL(sm_rglru_seg_reduce_kernel, grid, dim3(64), 0, (hipStream_t)stream, (float*)ab, s0,
+                       (const float*)a, (const float*)g, (const float*)state, (const int32_t*)cu,
+                       (const int32_t*)positions, (const int32_t*)slots, C, nseg);
+    DLLM_HIP_CHECK(hipGetLastError());
+    SM_DISPATCH(f32, sm_rglru_seg_scan_kernel, grid, dim3(64), 0, stream, (void*)out, (const float*)a, (const float*)g,
+                (const void*)y_raw, y_stride, (const void*)y_bias, (float*)state, (const float*)ab, (const float*)s0,
+                (const int32_t*)cu, (const int32_t*)slots, C, nseg);
+    return;
+  }
   SM_DISPATCH(f32, sm_rglru_scan_kernel, dim3((C + 63) / 64, seqs), dim3(64), 0, stream, (void*)out, (const float*)a,
               (const float*)g, (const void*)y_raw, y_stride, (const void*)y_bias, (float*)state, (const int32_t*)cu,
               (const int32_t*)positions, (const int32_t*)slots, C);

@@ -25,6 +25,8 @@ import torch
 from .. import _ext
 
 ACT_DTYPES = (torch.bfloat16, torch.float32)
+SCAN_SEGMENT = 128        # tokens per segment of the segmented RG-LRU scan (kSeg in seqmix.hip)
+SCAN_MIN_WAVES = 2048     # below this many (sequence, 64-channel) waves a long chunk is scanned in segments
 
 
 @dataclass
@@ -220,9 +222,15 @@ def rglru(u: torch.Tensor, y_raw: torch.Tensor, y_bias: torch.Tensor, ra_t: torc
     _k().sm_rglru_gates(a.data_ptr(), g.data_ptr(), u.data_ptr(), ra_t.data_ptr(), ra_b.data_ptr(), ri_t.data_ptr(),
                         ri_b.data_ptr(), lam.data_ptr(), t, nb, bw, float(decay_scale), f, _stream())
     out = torch.empty(t, c, dtype=act_dtype, device=u.device)
+    # few sequences with long chunks: the segmented two-launch scan (its waves = sequences x segments x
+    # C / 64); many sequences fill the chip with one wave per (sequence, 64 channels) already
+    ab = None
+    nseg = -(-sb.max_q_len // SCAN_SEGMENT)
+    if nseg > 1 and sb.num_seqs * (-(-c // 64)) < SCAN_MIN_WAVES:
+        ab = torch.empty(sb.num_seqs * (nseg * 2 + 1) * c, dtype=torch.float32, device=u.device)
     _k().sm_rglru_scan(out.data_ptr(), a.data_ptr(), g.data_ptr(), y_raw.data_ptr(), y_raw.stride(0),
                        y_bias.data_ptr(), state.data_ptr(), sb.cu.data_ptr(), sb.positions.data_ptr(),
-                       sb.state_slots.data_ptr(), sb.num_seqs, c, sb.max_q_len, f, _stream())
+                       sb.state_slots.data_ptr(), sb.num_seqs, c, sb.max_q_len, _ptr(ab), f, _stream())
     return out
 
 

@@ -231,7 +231,7 @@ def test_rglru_long_memory_across_portions(target, blocks):
     assert abs(a.min()) > 0.9          # decays are slow: position 0 matters at the end
     state = torch.full((3, c), 5.0, dtype=torch.float32, device=device)
     got, at = [], 0
-    for k in (2, 1, 64, 1, 1, 100, 3, 128):
+    for k in (2, 1, 64, 1, 1, 100, 3, 128):          # 128 at the end and 300 below: the segmented scan's sizes
         sb = _sb([(at, k)], device, [2])
         o = sm.rglru(torch.from_numpy(u[at:at + k]).to(device), yraw[at:at + k].to(device), yb.to(device),
                      ra.transpose(1, 2).contiguous().to(device), rab.to(device), ri.transpose(1, 2).contiguous().to(device),
@@ -239,6 +239,16 @@ def test_rglru_long_memory_across_portions(target, blocks):
         got.append(o.float().cpu().numpy())
         at += k
     assert at == n
+    np.testing.assert_allclose(np.concatenate(got), want, rtol=2e-4 if dtype == torch.float32 else 2e-2,
+                               atol=2e-5 if dtype == torch.float32 else 2e-2)
+    # the whole sequence in two portions of several segments each (the segmented two-launch scan on the
+    # GPU), the second continuing from the slot
+    got = []
+    for lo, k in ((0, 170), (170, 130)):
+        o = sm.rglru(torch.from_numpy(u[lo:lo + k]).to(device), yraw[lo:lo + k].to(device), yb.to(device),
+                     ra.transpose(1, 2).contiguous().to(device), rab.to(device), ri.transpose(1, 2).contiguous().to(device),
+                     rib.to(device), lam.to(device), state, _sb([(lo, k)], device, [1]), dtype)
+        got.append(o.float().cpu().numpy())
     np.testing.assert_allclose(np.concatenate(got), want, rtol=2e-4 if dtype == torch.float32 else 2e-2,
                                atol=2e-5 if dtype == torch.float32 else 2e-2)
 
