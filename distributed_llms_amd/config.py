@@ -22,7 +22,7 @@ from typing import Any, Dict, List, Optional
 @dataclass
 class ModelConfig:
     name: str
-    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2", "tudilix" (layer-list hybrid)
+    arch: str                      # "llama" (Llama-2/3), "mixtral", "gpt2"; layer-list models: "tudilix", "gikovik"
     vocab_size: int
     hidden_size: int
     intermediate_size: int
@@ -45,6 +45,10 @@ class ModelConfig:
     layers: Optional[List[Dict[str, Any]]] = None
     residual_mult: float = 1.0     # sublayer outputs enter the residual stream scaled by this
     logit_softcap: float = 0.0     # > 0: logits <- cap * tanh(logits / cap)
+    # arch "gikovik": {"start", "stop", "times"} -- layers [start, stop) are repeated ``times`` times back to back, sharing
+    # their weights (every repetition gets separate caches); and the width of the per-layer token input
+    loop: Optional[Dict[str, int]] = None
+    token_side_dim: int = 0
 
     # ------------------------------------------------------------------ sizes
     @property
@@ -54,6 +58,12 @@ class ModelConfig:
     @property
     def needs_state_slots(self) -> bool:
         """Sequences carry per-layer state besides paged K/V (recurrent state, convolution tails)."""
+        return self.layers is not None and self.arch == "tudilix"
+
+    @property
+    def needs_seq_index(self) -> bool:
+        """The stage's kernels take varlen metadata (each token's sequence index, chunk offsets) in
+        every step, decode steps included."""
         return self.layers is not None
 
     @property
@@ -75,8 +85,9 @@ class ModelConfig:
     def layer_param_count(self) -> int:
         h, i = self.hidden_size, self.intermediate_size
         if self.layers is not None:
-            from .models.hybrid import layer_param_count
-            return sum(layer_param_count(h, l) for l in self.layers) // max(1, len(self.layers))
+            from .models import stage_class
+            count = stage_class(self.arch).layer_param_count
+            return sum(count(h, l) for l in self.layers) // max(1, len(self.layers))
         attn = h * self.qkv_size + self.q_size * h
         if self.arch == "gpt2":
             attn += self.qkv_size + h  # biases
@@ -107,13 +118,21 @@ class ModelConfig:
 
     def kv_bytes_per_token(self, dtype_bytes: int = 2) -> int:
         if self.layers is not None:
-            from .models.hybrid import kv_width
-            return sum(kv_width(l) for l in self.layers) * dtype_bytes
+            from .models import stage_class
+            return stage_class(self.arch).kv_elements_per_token(self) * dtype_bytes
         return 2 * self.num_layers * self.kv_size * dtype_bytes
 
     # ----------------------------------------------------------- HF interop
     def to_hf_config(self) -> Dict[str, Any]:
         """A ``config.json``-compatible dict (written into ``shards/config.json``)."""
+        if self.arch == "gikovik":
+            d = {"architecture": "Gikovik", "layers": [dict(l) for l in self.layers], "norm": {"eps": self.norm_eps},
+                 "vocab": self.vocab_size, "width": self.hidden_size, "_dllm_name": self.name}
+            if self.loop:
+                d["loop"] = dict(self.loop)
+            if self.token_side_dim:
+                d["token_side"] = {"dim": self.token_side_dim}
+            return d
         if self.layers is not None:
             return {"architecture": "Tudilix", "layers": [dict(l) for l in self.layers],
                     "logit_softcap": self.logit_softcap, "norm": {"eps": self.norm_eps},
@@ -152,6 +171,8 @@ class ModelConfig:
     def from_hf_config(cfg: Dict[str, Any], name: Optional[str] = None) -> "ModelConfig":
         if cfg.get("architecture") == "Tudilix":
             return ModelConfig.from_layer_list(cfg, name)
+        if cfg.get("architecture") == "Gikovik":
+            return _from_gikovik(cfg, name)
         mt = cfg.get("model_type", "llama")
         name = name or cfg.get("_dllm_name") or cfg.get("_name_or_path") or mt
         eos = cfg.get("eos_token_id", 2)
@@ -209,6 +230,37 @@ def _from_layer_list(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelCo
 
 
 ModelConfig.from_layer_list = staticmethod(_from_layer_list)
+
+
+def _from_gikovik(cfg: Dict[str, Any], name: Optional[str] = None) -> ModelConfig:
+    """A ``config.json`` with "architecture": "Gikovik": ``width``, ``vocab``, ``norm.eps``, ``layers`` (per
+    layer ``type`` "latent_attention" | "latent_attention_2", ``mixer`` sizes, ``mlp`` None | dense | moe),
+    optionally ``loop`` (start, stop, times) and ``token_side.dim``."""
+    layers = [dict(l) for l in cfg["layers"]]
+    if not layers:
+        raise ValueError("layer-list config without layers")
+    for l in layers:
+        if l["type"] not in ("latent_attention", "latent_attention_2"):
+            raise ValueError(f"unsupported layer type {l['type']!r} (latent_attention, latent_attention_2)")
+        if l.get("mlp") is not None and l["mlp"].get("kind") not in ("dense", "moe"):
+            raise ValueError(f"unsupported mlp kind {l['mlp'].get('kind')!r} (dense, moe)")
+    extra = set(cfg.get("norm", {})) - {"eps"}
+    if extra:
+        raise ValueError(f"unsupported norm options {sorted(extra)}")
+    loop = cfg.get("loop")
+    if loop:
+        loop = {k: int(loop[k]) for k in ("start", "stop", "times")}
+        if not (0 <= loop["start"] < loop["stop"] <= len(layers)) or loop["times"] < 1:
+            raise ValueError(f"loop {loop} does not fit {len(layers)} layers")
+    mix = [l["mixer"] for l in layers]
+    ff = [l["mlp"]["ff"] if l["mlp"]["kind"] == "dense" else l["mlp"]["expert"]["ff"] for l in layers if l.get("mlp")]
+    return ModelConfig(
+        name=name or cfg.get("_dllm_name") or "gikovik", arch="gikovik", vocab_size=int(cfg["vocab"]),
+        hidden_size=int(cfg["width"]), intermediate_size=int(max(ff or [0])), num_layers=len(layers),
+        num_heads=max(m["heads"] for m in mix), num_kv_heads=1,
+        head_dim=max(m["kv_rank"] + m.get("rot_dim", 0) for m in mix), max_position=1 << 30,
+        norm_eps=float(cfg["norm"]["eps"]), bos_token_id=-1, eos_token_id=-1, layers=layers, loop=loop or None,
+        token_side_dim=int((cfg.get("token_side") or {}).get("dim", 0)))
 
 
 _LLAMA3_ROPE = {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
@@ -269,6 +321,21 @@ PRESETS: Dict[str, ModelConfig] = {
                         "scaling": {"factor": 8.0, "fast": 16.0, "original": 512, "slow": 2.0}}},
              "mlp": None},
         ]}, name="tiny-tudilix"),
+    "tiny-gikovik": _from_gikovik({
+        "architecture": "Gikovik", "vocab": 320, "width": 128, "norm": {"eps": 1e-5}, "token_side": {"dim": 16},
+        "loop": {"start": 1, "stop": 3, "times": 2},
+        "layers": [
+            {"type": "latent_attention", "mixer": {"dim": 16, "heads": 4, "kv_rank": 48, "q_rank": 64, "scale": 0.25,
+                                                   "vdim": 24},
+             "mlp": {"kind": "dense", "ff": 192}},
+            {"type": "latent_attention_2", "mixer": {"dim": 32, "heads": 2, "kv_rank": 40, "q_rank": 48,
+                                                     "rot": {"base": 10000.0, "dims": 8}, "rot_dim": 8, "scale": 0.15,
+                                                     "vdim": 32},
+             "mlp": {"kind": "moe", "expert": {"ff": 64}, "shared": {"ff": 32},
+                     "router": {"experts": 6, "groups": {"count": 3, "keep": 2}, "scale": 1.5, "top": 2}}},
+            {"type": "latent_attention", "mixer": {"dim": 16, "heads": 4, "kv_rank": 48, "q_rank": 64, "scale": 0.25,
+                                                   "vdim": 24}, "mlp": None},
+        ]}, name="tiny-gikovik"),
     "tiny-gpt2": ModelConfig(
         name="tiny-gpt2", arch="gpt2", vocab_size=512, hidden_size=128,
         intermediate_size=512, num_layers=4, num_heads=2, num_kv_heads=2, head_dim=64,

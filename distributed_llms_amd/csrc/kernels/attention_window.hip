@@ -2,7 +2,8 @@
 // (ops/seqmix.py window_attention): caches k [NB, G, BS, D] (one row per key), v [NB, G, Dv, BS]
 // (transposed inside a block: 8 keys of one value channel are one 16-byte load),
 // query head h reads K/V head h / (H / G), a query at position p sees the keys j of its sequence with
-// 0 <= p - j < window.  Scores, softmax weights and the weighted sum are float32; T is the storage
+// 0 <= p - j < window; `sinks` (float32 [H], or null) adds exp(sink_h) to head h's softmax denominator
+// (a learned per-head logit that takes part in the normalisation only).  Scores, softmax weights and the weighted sum are float32; T is the storage
 // type (bf16 or float).  Head sizes, window and block size are runtime values.
 //
 //   window_attn_row_kernel   one workgroup per (query token, head): keys in tiles of 256, one key per
@@ -76,7 +77,7 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
     void* __restrict__ out_, const void* __restrict__ q_, const void* __restrict__ k_cache_,
     const void* __restrict__ v_cache_, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int t0, int H, int G, int D, int Dv,
-    int bs, int window, float scale) {
+    int bs, int window, float scale, const float* __restrict__ sinks) {
   extern __shared__ float lds[];
   float* qs = lds;                       // [D]
   float* p = qs + D;                     // [kWinTile]
@@ -132,6 +133,12 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
     }
     __syncthreads();                            // before the next tile overwrites p and rows
   }
+  // a sink adds exp(sink) to the denominator; nothing is attended to through it
+  float fin = 1.0f / l;
+  if (sinks) {
+    const float sk = sinks[h], mf = fmaxf(m, sk), cf = expf(m - mf);
+    fin = cf / (l * cf + expf(sk - mf));
+  }
   // sum the key subgroups
   T* out = (T*)out_ + ((size_t)t * H + h) * Dv;
 #pragma unroll
@@ -142,7 +149,7 @@ __global__ void __launch_bounds__(kWinTile) window_attn_row_kernel(
     if (sub == 0 && e < Dv) {
       float a = 0.f;
       for (int s2 = 0; s2 < nsub; ++s2) a += part[s2 * Dv + e];
-      out[e] = (T)(a / l);
+      out[e] = (T)(a * fin);
     }
     __syncthreads();
   }
@@ -155,7 +162,7 @@ static size_t win_row_lds(int D, int Dv) {
 
 static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t positions, uintptr_t tok_seq, int t0, int rows, int H, int G, int D,
-                        int Dv, int bs, int window, float scale, int f32, uintptr_t stream) {
+                        int Dv, int bs, int window, float scale, uintptr_t sinks, int f32, uintptr_t stream) {
   DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && D > 0 && Dv > 0 && Dv <= kWinTile * kWinMaxAcc, "window attention heads");
   DLLM_HOST_CHECK(bs > 0 && window >= 1 && max_blocks > 0 && H <= 65535, "window attention sizes");
   const size_t lds = win_row_lds(D, Dv);
@@ -164,12 +171,12 @@ static void launch_rows(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t
     hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_row_kernel<float>), dim3(rows, H), dim3(kWinTile), lds,
                        (hipStream_t)stream, (void*)out, (const void*)q, (const void*)k_cache, (const void*)v_cache,
                        (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, t0,
-                       H, G, D, Dv, bs, window, scale);
+                       H, G, D, Dv, bs, window, scale, (const float*)sinks);
   else
     hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_row_kernel<bf16>), dim3(rows, H), dim3(kWinTile), lds,
                        (hipStream_t)stream, (void*)out, (const void*)q, (const void*)k_cache, (const void*)v_cache,
                        (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, t0,
-                       H, G, D, Dv, bs, window, scale);
+                       H, G, D, Dv, bs, window, scale, (const float*)sinks);
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
@@ -193,10 +200,10 @@ __device__ __forceinline__ void split_pack(const float (&e)[8], bf16x8& ph, bf16
 }
 
 // --------------------------------------------------------------------------- MFMA prompt kernel (bf16)
-constexpr int kQT = 1;           // MFMA column tiles (16 queries) per wave: 1 keeps the kernel at <= 128 VGPRs
-                                 // (4 waves per SIMD, so one wave's softmax overlaps another's MFMAs); 2 halves the
-                                 // LDS reads per MFMA but measured slower at 1 wave per SIMD
-constexpr int kTQ = 64 * kQT;    // queries per workgroup: 4 waves x kQT column tiles
+// QT (template): MFMA column tiles (16 queries) per wave.  1 keeps heads up to 128 wide at <= 128 VGPRs
+// (4 waves per SIMD, so one wave's softmax overlaps another's MFMAs; 2 measured slower there at 1 wave
+// per SIMD).  2 halves the LDS reads per MFMA: every K / V^T fragment a wave reads feeds both of its
+// column tiles.  A workgroup has 4 waves x QT column tiles = 64 QT queries.
 constexpr int kTK = 32;          // keys per tile
 constexpr int kPad = 8;          // bf16 elements of row padding in LDS (16 bytes: rows start on different banks)
 constexpr float kLog2e = 1.4426950408889634f;
@@ -204,12 +211,13 @@ constexpr float kLog2e = 1.4426950408889634f;
 // NQK: 32-wide K-dim steps of q.k (D <= 32 NQK); NDV: 16-wide tiles of value channels (Dv <= 16 NDV).
 // Every K / V^T fragment a wave reads from LDS feeds both of its query column tiles; the next key tile's
 // global loads are issued before the current tile's MFMAs and land in LDS after them.
-template <int NQK, int NDV>
+template <int NQK, int NDV, int QT>
 __global__ void __launch_bounds__(256) window_attn_tile_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ cu, const int32_t* __restrict__ positions, int seq0, int nseq, int nqt, int H, int G,
-    int D, int Dv, int bs, int window, float scale) {
+    int D, int Dv, int bs, int window, float scale, const float* __restrict__ sinks, int sub) {
+  constexpr int kQT = QT, kTQ = 64 * QT;
   constexpr int DP = 32 * NQK, KROW = DP + kPad, VROW = kTK + kPad;
   constexpr int KPT = (kTK * (DP / 8) + 255) / 256, VPT = (16 * NDV * (kTK / 8) + 255) / 256;   // 16-byte pieces per thread
   __shared__ __attribute__((aligned(16))) bf16 ks[kTK * KROW];          // K tile, key j at row krow32(j)
@@ -217,11 +225,15 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   // Workgroups are dealt to the 8 XCDs round-robin by their linear id.  The id is decoded so that
   // every tile that reads one (sequence, K/V head) pair -- all its query tiles and the heads of the
   // group -- runs on the same XCD, whose L2 then serves the re-reads of that pair's keys and values;
-  // within a pair the longest query tiles (most keys, causal) start first.
+  // within a pair the longest query tiles (most keys, causal) start first.  With fewer pairs than XCDs
+  // (few sequences that share one K/V head) a pair's tiles are dealt to `sub` XCDs in turn, so that no
+  // XCD stays idle.
   const int R = H / G, per_pair = nqt * R, pairs = nseq * G;
+  const int per_part = (per_pair + sub - 1) / sub;
   const int xcd = blockIdx.x & 7, slot = blockIdx.x >> 3;
-  const int pair = (slot / per_pair) * 8 + xcd, rem = slot % per_pair;
-  if (pair >= pairs) return;
+  const int vpair = (slot / per_part) * 8 + xcd;
+  const int pair = vpair / sub, rem = (slot % per_part) * sub + vpair % sub;
+  if (pair >= pairs || rem >= per_pair) return;
   const int b = seq0 + pair / G, g = pair % G;
   const int h = g * R + rem % R;
   const int lo_t = cu[b], n = cu[b + 1] - lo_t;
@@ -401,7 +413,11 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
 #pragma unroll
   for (int c2 = 0; c2 < kQT; ++c2) {
     if (!qok[c2]) continue;
-    const float inv = 1.0f / l[c2];
+    float inv = 1.0f / l[c2];
+    if (sinks) {                                   // exp(sink) joins the denominator (scores here are in log2 units)
+      const float sk = sinks[h] * kLog2e, mf = fmaxf(m[c2], sk), cf = __builtin_amdgcn_exp2f(m[c2] - mf);
+      inv = cf / (l[c2] * cf + __builtin_amdgcn_exp2f(sk - mf));
+    }
     bf16* orow = out + ((size_t)(lo_t + ql[c2]) * H + h) * Dv;
 #pragma unroll
     for (int dt = 0; dt < NDV; ++dt) {
@@ -416,23 +432,26 @@ __global__ void __launch_bounds__(256) window_attn_tile_kernel(
   }
 }
 
-template <int NQK, int NDV>
+template <int NQK, int NDV, int QT>
 static void launch_tile(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                         int max_blocks, uintptr_t cu, uintptr_t positions, int seq0, int nseq, int max_q_len, int H,
-                        int G, int D, int Dv, int bs, int window, float scale, uintptr_t stream) {
+                        int G, int D, int Dv, int bs, int window, float scale, uintptr_t sinks, uintptr_t stream) {
+  constexpr int kTQ = 64 * QT;
   const int nqt = (max_q_len + kTQ - 1) / kTQ;
-  const long per_xcd = (long)((nseq * G + 7) / 8) * nqt * (H / G);      // workgroups of one XCD
+  const int pairs = nseq * G, per_pair = nqt * (H / G);
+  const int sub = pairs < 8 ? 8 : 1;                                    // XCDs that share a pair's tiles
+  const long per_xcd = (long)(((long)pairs * sub + 7) / 8) * ((per_pair + sub - 1) / sub);   // workgroups of one XCD
   DLLM_HOST_CHECK(per_xcd * 8 < (1L << 31), "window attention grid");
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV>), dim3((unsigned)(per_xcd * 8)),
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_tile_kernel<NQK, NDV, QT>), dim3((unsigned)(per_xcd * 8)),
                      dim3(256), 0, (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache,
                      (const bf16*)v_cache, (const int32_t*)block_tables, max_blocks, (const int32_t*)cu,
-                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, scale);
+                     (const int32_t*)positions, seq0, nseq, nqt, H, G, D, Dv, bs, window, scale, (const float*)sinks, sub);
   DLLM_HIP_CHECK(hipGetLastError());
 }
 
 // --------------------------------------------------------------------------- MFMA decode kernel (bf16)
-// One workgroup per (one-token sequence, K/V head): the 16 MFMA columns are the query heads of the
-// group, so the keys and values of a K/V head are read once for all of them.  The wave's key tiles
+// One workgroup per (one-token sequence, K/V head, 16 query heads of its group): the 16 MFMA columns are
+// query heads of the group, so the keys and values of a K/V head are read once for 16 of them.  The wave's key tiles
 // (32 keys, tile index mod kDW = wave) go from global memory straight into MFMA fragments: K rows as
 // the A operand of S^T = K Q^T (row r of a 16-key half holds the key that makes the accumulator hand
 // each lane 8 consecutive keys), V^T pieces (8 keys of one channel, 16 bytes) as the A operand of
@@ -444,12 +463,16 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
     bf16* __restrict__ out, const bf16* __restrict__ q, const bf16* __restrict__ k_cache,
     const bf16* __restrict__ v_cache, const int32_t* __restrict__ block_tables, int max_blocks,
     const int32_t* __restrict__ positions, const int32_t* __restrict__ tok_seq, int H, int G, int D, int Dv, int bs,
-    int window, float scale) {
+    int window, float scale, const float* __restrict__ sinks, int hpw, int splits, float* __restrict__ ws) {
   constexpr int DVP = 16 * NDV;
   __shared__ float so[kDW][16][DVP + 1];
   __shared__ float sml[kDW][2][16];
-  const int t = blockIdx.x, g = blockIdx.y;
-  const int R = H / G;
+  // the query heads of a K/V head are dealt to workgroups hpw (<= 16) at a time: part p runs heads
+  // hpw p .. of the group (fewer heads per workgroup when few rows would leave most CUs idle)
+  const int t = blockIdx.x;
+  const int R = H / G, parts = (R + hpw - 1) / hpw;
+  const int g = blockIdx.y / parts, part = blockIdx.y - g * parts;
+  const int hb = g * R + hpw * part, nh = min(hpw, R - hpw * part);    // first head and heads of this workgroup
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, col = lane & 15, grp = lane >> 4;
   const int pos = positions[t], b = tok_seq[t];
   const int lo = max(0, pos - window + 1);
@@ -457,14 +480,14 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
   const int32_t* bt = block_tables + (size_t)b * max_blocks;
   bf16x8 qf[NQK];
   {
-    const bf16* qrow = q + ((size_t)t * H + g * R + min(col, R - 1)) * D;
+    const bf16* qrow = q + ((size_t)t * H + hb + min(col, nh - 1)) * D;
 #pragma unroll
     for (int s2 = 0; s2 < NQK; ++s2) {
       const int d0 = 32 * s2 + 8 * grp;
       bf16x8 v;
 #pragma unroll
       for (int j = 0; j < 8; ++j) v[j] = (bf16)0.f;
-      if (d0 + 8 <= D && col < R) v = *reinterpret_cast<const bf16x8*>(qrow + d0);
+      if (d0 + 8 <= D && col < nh) v = *reinterpret_cast<const bf16x8*>(qrow + d0);
       qf[s2] = v;
     }
   }
@@ -490,9 +513,13 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
       }
     }
   };
-  const int kbeg = (lo & ~31) + 32 * wave;
-  if (kbeg <= pos) load_k(kbeg);
-  for (int k0 = kbeg; k0 <= pos; k0 += 32 * kDW) {
+  // the row's 32-key tiles are cut into `splits` runs, one per workgroup along z (long contexts of few
+  // rows: the partial results meet in window_attn_merge_kernel); inside a run, tile index mod kDW = wave
+  const int k00 = lo & ~31, ntile = ((pos - k00) >> 5) + 1, tps = (ntile + splits - 1) / splits;
+  const int kstop = k00 + 32 * min(ntile, ((int)blockIdx.z + 1) * tps);
+  const int kbeg = k00 + 32 * ((int)blockIdx.z * tps + wave);
+  if (kbeg < kstop) load_k(kbeg);
+  for (int k0 = kbeg; k0 < kstop; k0 += 32 * kDW) {
     // this tile's V^T pieces (8 keys from k0 + 8 grp, clamped to the last piece that exists) go out first
     const int kp8 = min(k0 + 8 * grp, pos & ~7);
     const bf16* vbase = v_cache + ((size_t)bt[kp8 >> bsh] * G + g) * Dv * bs + (kp8 & (bs - 1));
@@ -513,7 +540,7 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
       }
     }
     // the wave's next tile's K rows are in flight during this tile's softmax and P.V
-    if (k0 + 32 * kDW <= pos) load_k(k0 + 32 * kDW);
+    if (k0 + 32 * kDW < kstop) load_k(k0 + 32 * kDW);
     float p[8];
     float cm = -INFINITY;
 #pragma unroll
@@ -553,31 +580,85 @@ __global__ void __launch_bounds__(64 * kDW) window_attn_decode_kernel(
 #pragma unroll
     for (int i = 0; i < 4; ++i) so[wave][col][16 * dt + 4 * grp + i] = acc[dt][i];
   __syncthreads();
-  for (int idx = tid; idx < R * Dv; idx += 64 * kDW) {
+  for (int idx = tid; idx < nh * Dv; idx += 64 * kDW) {
     const int hh = idx / Dv, e = idx - hh * Dv;
     float mm = -INFINITY;
 #pragma unroll
     for (int w = 0; w < kDW; ++w) mm = fmaxf(mm, sml[w][0][hh]);
     float ll = 0.f, o = 0.f;
+    if (splits > 1) {                              // unnormalised partial: Dv sums, then their maximum and weight
+#pragma unroll
+      for (int w = 0; w < kDW; ++w) {
+        const float f = sml[w][0][hh] == -INFINITY ? 0.f : expf(sml[w][0][hh] - mm);
+        ll += sml[w][1][hh] * f;
+        o += so[w][hh][e] * f;
+      }
+      float* part = ws + (((size_t)t * H + hb + hh) * splits + blockIdx.z) * (Dv + 2);
+      part[e] = o;
+      if (e == 0) part[Dv] = mm, part[Dv + 1] = ll;
+      continue;
+    }
+    if (sinks) {                                   // exp(sink) joins the denominator
+      const float sk = sinks[hb + hh];
+      mm = fmaxf(mm, sk);
+      ll = expf(sk - mm);
+    }
 #pragma unroll
     for (int w = 0; w < kDW; ++w) {
       const float f = sml[w][0][hh] == -INFINITY ? 0.f : expf(sml[w][0][hh] - mm);
       ll += sml[w][1][hh] * f;
       o += so[w][hh][e] * f;
     }
-    out[((size_t)t * H + g * R + hh) * Dv + e] = (bf16)(o / ll);
+    out[((size_t)t * H + hb + hh) * Dv + e] = (bf16)(o / ll);
+  }
+}
+
+// Sum of a row's partial results over the context splits: ws [rows, H, splits, Dv + 2] (Dv unnormalised
+// sums relative to the split's maximum, the maximum, the weight sum) -> out [rows, H, Dv]
+__global__ void __launch_bounds__(64) window_attn_merge_kernel(bf16* __restrict__ out, const float* __restrict__ ws,
+                                                               int H, int Dv, int splits,
+                                                               const float* __restrict__ sinks) {
+  const int t = blockIdx.x, h = blockIdx.y;
+  const float* part = ws + ((size_t)t * H + h) * splits * (Dv + 2);
+  float mm = sinks ? sinks[h] : -INFINITY;
+  for (int s2 = 0; s2 < splits; ++s2) mm = fmaxf(mm, part[s2 * (Dv + 2) + Dv]);
+  float ll = sinks ? expf(sinks[h] - mm) : 0.f;
+  for (int s2 = 0; s2 < splits; ++s2) {
+    const float m = part[s2 * (Dv + 2) + Dv];
+    if (m != -INFINITY) ll += part[s2 * (Dv + 2) + Dv + 1] * expf(m - mm);
+  }
+  for (int e = threadIdx.x; e < Dv; e += 64) {
+    float o = 0.f;
+    for (int s2 = 0; s2 < splits; ++s2) {
+      const float m = part[s2 * (Dv + 2) + Dv];
+      if (m != -INFINITY) o += part[s2 * (Dv + 2) + e] * expf(m - mm);
+    }
+    out[((size_t)t * H + h) * Dv + e] = (bf16)(o / ll);
   }
 }
 
 template <int NQK, int NDV>
 static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                           int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
-                          int Dv, int bs, int window, float scale, uintptr_t stream) {
-  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_decode_kernel<NQK, NDV>), dim3(rows, G), dim3(64 * kDW), 0,
+                          int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
+                          uintptr_t stream) {
+  // heads per workgroup: 16 (all MFMA columns) when rows x K/V heads fill the chip, else halved until
+  // about half the CUs have a workgroup -- the keys are re-read from L2, the columns left idle cost nothing
+  const int R = H / G;
+  int hpw = std::min(16, R);
+  while (hpw > 2 && (long)rows * G * ((R + hpw - 1) / hpw) < 128) hpw = (hpw + 1) / 2;
+  splits = ws ? std::max(1, std::min(splits, 64)) : 1;
+  hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_decode_kernel<NQK, NDV>),
+                     dim3(rows, G * ((R + hpw - 1) / hpw), splits), dim3(64 * kDW), 0,
                      (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,
                      (const int32_t*)block_tables, max_blocks, (const int32_t*)positions, (const int32_t*)tok_seq, H, G,
-                     D, Dv, bs, window, scale);
+                     D, Dv, bs, window, scale, (const float*)sinks, hpw, splits, (float*)ws);
   DLLM_HIP_CHECK(hipGetLastError());
+  if (splits > 1) {
+    hipLaunchKernelGGL(window_attn_merge_kernel, dim3(rows, H), dim3(64), 0, (hipStream_t)stream, (bf16*)out,
+                       (const float*)ws, H, Dv, splits, (const float*)sinks);
+    DLLM_HIP_CHECK(hipGetLastError());
+  }
 }
 
 // bf16 with 16-byte rows and pieces goes to the matrix cores; float32 (the exact path), odd head sizes
@@ -587,16 +668,19 @@ static bool win_mfma_ok(int f32, int H, int G, int D, int Dv, int bs) {
          H % G == 0;
 }
 
-// Decode rows: tokens [0, rows) are one-token sequences.
+// Decode rows: tokens [0, rows) are one-token sequences.  `splits` > 1 with `ws` (float32
+// [rows, H, splits, Dv + 2]) cuts every row's keys into that many runs on separate workgroups (the MFMA
+// kernel only; the row kernel ignores it).
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
-                           int Dv, int bs, int window, float scale, int f32, uintptr_t stream) {
+                           int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
+                           int f32, uintptr_t stream) {
   if (rows <= 0) return;
-  if (win_mfma_ok(f32, H, G, D, Dv, bs) && H / G <= 16 && G <= 65535) {
+  if (win_mfma_ok(f32, H, G, D, Dv, bs) && (long)G * ((H / G + 1) / 2) <= 65535) {
     DLLM_HOST_CHECK(window >= 1 && max_blocks > 0, "window attention sizes");
 #define WIN_DEC(NQK, NDV)                                                                                       \
   launch_decode<NQK, NDV>(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, rows, H, G, D, Dv, \
-                          bs, window, scale, stream)
+                          bs, window, scale, sinks, splits, ws, stream)
     if (D <= 64 && Dv <= 64) WIN_DEC(2, 4);
     else if (D <= 128 && Dv <= 128) WIN_DEC(4, 8);
     else WIN_DEC(8, 16);
@@ -604,31 +688,31 @@ void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintpt
     return;
   }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, 0, rows, H, G, D, Dv, bs, window,
-              scale, f32, stream);
+              scale, sinks, f32, stream);
 }
 
 // Prompt chunks: tokens [t0 .. tokens) of sequences [seq0, seqs).
 void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                             int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
                             int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, float scale,
-                            int f32, uintptr_t stream) {
+                            uintptr_t sinks, int f32, uintptr_t stream) {
   // tokens of the decode rows come first: one per sequence before seq0
   const int t0 = seq0;
   if (tokens <= t0) return;
   if (win_mfma_ok(f32, H, G, D, Dv, bs) && seqs > seq0 && max_q_len > 1) {
     DLLM_HOST_CHECK(H > 0 && G > 0 && H % G == 0 && H <= 65535 && seqs - seq0 <= 65535, "window attention heads");
     DLLM_HOST_CHECK(bs > 0 && window >= 1 && max_blocks > 0, "window attention sizes");
-#define WIN_TILE(NQK, NDV)                                                                                  \
-  launch_tile<NQK, NDV>(out, q, k_cache, v_cache, block_tables, max_blocks, cu, positions, seq0, seqs - seq0, \
-                        max_q_len, H, G, D, Dv, bs, window, scale, stream)
-    if (D <= 64 && Dv <= 64) WIN_TILE(2, 4);
-    else if (D <= 128 && Dv <= 128) WIN_TILE(4, 8);
-    else WIN_TILE(8, 16);
+#define WIN_TILE(NQK, NDV, QT)                                                                                  \
+  launch_tile<NQK, NDV, QT>(out, q, k_cache, v_cache, block_tables, max_blocks, cu, positions, seq0, seqs - seq0, \
+                            max_q_len, H, G, D, Dv, bs, window, scale, sinks, stream)
+    if (D <= 64 && Dv <= 64) WIN_TILE(2, 4, 1);
+    else if (D <= 128 && Dv <= 128) WIN_TILE(4, 8, 1);
+    else WIN_TILE(8, 16, 2);     // wide heads: 2b-size latent attention prompts 32 x 1024 +7 %, 4 x 4096 +29 % over QT = 1
 #undef WIN_TILE
     return;
   }
   launch_rows(out, q, k_cache, v_cache, block_tables, max_blocks, positions, tok_seq, t0, tokens - t0, H, G, D, Dv, bs,
-              window, scale, f32, stream);
+              window, scale, sinks, f32, stream);
 }
 
 }  // namespace dllm

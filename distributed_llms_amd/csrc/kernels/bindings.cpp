@@ -49,6 +49,17 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("sm_attn_prep", &dllm::sm_attn_prep);
   m.def("sm_window_attn_decode", &dllm::sm_window_attn_decode);
   m.def("sm_window_attn_prefill", &dllm::sm_window_attn_prefill);
+  m.def("lat_prep", &dllm::lat_prep);
+  m.def("lat_q_pack", &dllm::lat_q_pack);
+  m.def("lat_head_gate", &dllm::lat_head_gate);
+  m.def("par_add", &dllm::par_add);
+  m.def("stream_cat", &dllm::stream_cat);
+  m.def("stream_set", &dllm::stream_set);
+  m.def("side_gate", &dllm::side_gate);
+  m.def("silu_glu", &dllm::silu_glu);
+  m.def("moe_route_groups", &dllm::moe_route_groups);
+  m.def("relu_sq", &dllm::relu_sq);
+  m.def("moe_combine_gated", &dllm::moe_combine_gated);
   m.def("p2p_inbox_bytes", &dllm::p2p_inbox_bytes);
   m.def("p2p_standin", &dllm::p2p_standin);
   m.def("p2p_host_words", &dllm::p2p_host_words);

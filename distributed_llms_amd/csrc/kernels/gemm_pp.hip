@@ -148,7 +148,8 @@ __device__ __forceinline__ int pp_b_row(int r, int n_t, int half) {
 }
 }  // namespace
 
-// MODE 0: C bf16 [M, N];  1: split-K slab P (f16 x 2^-6, common.h) [S, M, N];  2: SwiGLU C [M, N/2].
+// MODE 0: C bf16 [M, N];  1: split-K slab P (f16 x 2^-6, common.h) [S, M, N];  2: SwiGLU C [M, N/2];
+// 3: C = max(A B^T, 0)^2 (the activation of two-matrix experts, in the epilogue).
 // VAR bit 0: weights nontemporal (read once); bit 1: grouped row-tile order (prefill, no split).
 template <int BN, int MODE, int VAR>
 __global__ void __launch_bounds__(256, 1) gemm_pp_kernel(const bf16* __restrict__ A, const bf16* __restrict__ B,
@@ -574,7 +575,14 @@ __global__ void __launch_bounds__(256, 1) gemm_pp_kernel(const bf16* __restrict_
         } else {
           bf16x4 h;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) h[e] = f2bf(v[e]);
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (MODE == 3) {
+              const float p = fmaxf(v[e], 0.f);
+              h[e] = f2bf(p * p);
+            } else {
+              h[e] = f2bf(v[e]);
+            }
+          }
           *reinterpret_cast<bf16x4*>(smem + row * OPITCH + col) = h;
         }
       }
@@ -704,7 +712,7 @@ void gemm_pp_moe(uintptr_t y, uintptr_t x, uintptr_t gather, uintptr_t w, uintpt
   DLLM_HOST_CHECK(E >= 1 && E <= 256, "1 <= experts <= 256");
   DLLM_HOST_CHECK(K % PBK == 0 && K >= PBK, "K must be a positive multiple of 64");
   DLLM_HOST_CHECK(N % 256 == 0, "N must be a multiple of 256");
-  DLLM_HOST_CHECK(mode == 0 || mode == 1, "mode 0 (plain) or 1 (SwiGLU)");
+  DLLM_HOST_CHECK(mode == 0 || mode == 1 || mode == 2, "mode 0 (plain), 1 (SwiGLU) or 2 (squared ReLU)");
   DLLM_HOST_CHECK(xrows >= 1 && slots >= 1, "rows");
   DLLM_HOST_CHECK((long)xrows * K * 2 < (1L << 32) && (long)N * K * 2 < (1L << 32), "operands must be < 4 GiB");
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
@@ -712,6 +720,10 @@ void gemm_pp_moe(uintptr_t y, uintptr_t x, uintptr_t gather, uintptr_t w, uintpt
   DLLM_HOST_CHECK(grid < (1L << 31), "grid");
   if (mode == 1)
     hipLaunchKernelGGL((gemm_pp_kernel<256, 2, 128 | 32 | 2>), dim3((unsigned)grid), dim3(256), 0, s, (const bf16*)x,
+                       (const bf16*)w, (bf16*)y, (float*)nullptr, xrows, N, K, K / PBK, 1, (float*)nullptr,
+                       (const int*)gather, (const int*)counts, (const int*)offsets, E);
+  else if (mode == 2)
+    hipLaunchKernelGGL((gemm_pp_kernel<256, 3, 128 | 32 | 2>), dim3((unsigned)grid), dim3(256), 0, s, (const bf16*)x,
                        (const bf16*)w, (bf16*)y, (float*)nullptr, xrows, N, K, K / PBK, 1, (float*)nullptr,
                        (const int*)gather, (const int*)counts, (const int*)offsets, E);
   else

@@ -74,7 +74,7 @@ void sm_embed_f32(uintptr_t out, uintptr_t ids, uintptr_t table, int tokens, int
 void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, float eps, float offset, int f32,
                  uintptr_t stream);
 void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
-                      int rows, int width, float eps, float mult, int f32, uintptr_t stream);
+                      int rows, int width, float eps, float mult, float offset, int f32, uintptr_t stream);
 void sm_causal_conv(uintptr_t y, uintptr_t u, long stride, uintptr_t w, uintptr_t bias, uintptr_t in_bias,
                     uintptr_t state, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, uintptr_t slots,
                     int tokens, int seqs, int C, int taps, int f32, int out_f32, uintptr_t stream);
@@ -94,11 +94,34 @@ void sm_attn_prep(uintptr_t q_out, uintptr_t qkv, uintptr_t conv_w, uintptr_t st
                   uintptr_t stream);
 void sm_window_attn_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                            int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
-                           int Dv, int bs, int window, float scale, int f32, uintptr_t stream);
+                           int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
+                           int f32, uintptr_t stream);
 void sm_window_attn_prefill(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr_t v_cache, uintptr_t block_tables,
                             int max_blocks, uintptr_t cu, uintptr_t positions, uintptr_t tok_seq, int seq0, int seqs,
                             int tokens, int max_q_len, int H, int G, int D, int Dv, int bs, int window, float scale,
-                            int f32, uintptr_t stream);
+                            uintptr_t sinks, int f32, uintptr_t stream);
+// latent attention input stage and parallel layers on a float32 stream (latent.hip)
+void lat_prep(uintptr_t cq, uintptr_t down, long ld, int q_off, int q_rank, uintptr_t qn_w, int c_off, int rank,
+              uintptr_t cn_w, int r_off, int rot_dim, uintptr_t freqs, int nfreq, uintptr_t positions,
+              uintptr_t slot_mapping, uintptr_t k_cache, uintptr_t v_cache, int bs, float eps, int tokens, int f32,
+              uintptr_t stream);
+void lat_q_pack(uintptr_t out, uintptr_t qa, uintptr_t q, int tokens, int H, int rank, int dim, int rot_dim,
+                uintptr_t freqs, int nfreq, uintptr_t positions, int f32, uintptr_t stream);
+void lat_head_gate(uintptr_t out, uintptr_t o, uintptr_t gate, long ld, int tokens, int H, int vdim, int f32,
+                   uintptr_t stream);
+void par_add(uintptr_t x, uintptr_t a, uintptr_t b, uintptr_t x_rounded, long n, int f32, uintptr_t stream);
+void stream_cat(uintptr_t out, uintptr_t x, uintptr_t x0, int rows, int width, int f32, uintptr_t stream);
+void stream_set(uintptr_t x, uintptr_t a, long n, int f32, uintptr_t stream);
+void silu_glu(uintptr_t out, uintptr_t gu, int tokens, int F, int f32, uintptr_t stream);
+void side_gate(uintptr_t g, uintptr_t z, uintptr_t table, uintptr_t ids, int tokens, int vocab, int total, int off,
+               int dim, int f32, uintptr_t stream);
+// grouped-choice router, squared ReLU and the weighted sum with a gated shared expert (moe.hip)
+void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, int E, int k, int groups, int keep,
+                      float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts, uintptr_t offsets,
+                      uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream);
+void relu_sq(uintptr_t y, long n, int f32, uintptr_t stream);
+void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,
+                       uintptr_t gate_logits, long gate_ld, int T, int H, int k, int f32, uintptr_t stream);
 
 long p2p_inbox_bytes(long chunk, int nslots);
 void p2p_standin(uintptr_t src, uintptr_t s_inbox, long s_bytes, uint64_t s_seq0, uintptr_t dst, uintptr_t r_inbox,

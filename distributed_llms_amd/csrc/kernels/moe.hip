@@ -11,6 +11,7 @@
 //  moe_combine  : out[t] = sum_j w[t,j] * y[inv[t,j]]   (fixed j order: deterministic)
 #include "skinny_common.h"
 #include "launchers.h"
+#include "stream_common.h"
 
 namespace dllm {
 
@@ -175,6 +176,7 @@ __global__ void __launch_bounds__(1024) moe_scatter_kernel(const int* __restrict
 
 constexpr int MOE_EPI_STORE = 0;
 constexpr int MOE_EPI_SWIGLU = 1;
+constexpr int MOE_EPI_RELU2 = 2;          // store max(v, 0)^2: the activation of two-matrix experts
 
 // Rows [0, cnt) of one expert in chunks of MT*16 rows; every chunk streams the WG's W column
 // tile once (K split over the WAVES waves, partial tiles summed through LDS).
@@ -207,7 +209,9 @@ __device__ __forceinline__ void moe_rows(float* red, bf16* __restrict__ y, const
     } else {
       for (int q = threadIdx.x; q < rows * BN; q += NTHR) {
         const int m = q / BN, c = q % BN;
-        y[(size_t)(off + r0 + m) * ldy + blockIdx.x * BN + c] = f2bf(red[m * BN + c]);
+        float v = red[m * BN + c];
+        if (EPI == MOE_EPI_RELU2) v = fmaxf(v, 0.f) * fmaxf(v, 0.f);
+        y[(size_t)(off + r0 + m) * ldy + blockIdx.x * BN + c] = f2bf(v);
       }
     }
     __syncthreads();
@@ -313,6 +317,10 @@ static void launch_grouped(hipStream_t s, bf16* y, const bf16* x, const int* gat
     DLLM_HOST_CHECK(N % BN == 0, "moe grouped: 2I must be a multiple of the column tile");
     hipLaunchKernelGGL((moe_grouped_kernel<MTMAX, NT, WAVES, MOE_EPI_SWIGLU>), dim3(N / BN, E), dim3(WAVES * 64), 0,
                        s, y, x, gather, w, counts, offsets, N, K, N / 2);
+  } else if (mode == 2) {
+    DLLM_HOST_CHECK(N % BN == 0, "moe grouped: N must be a multiple of the column tile");
+    hipLaunchKernelGGL((moe_grouped_kernel<MTMAX, NT, WAVES, MOE_EPI_RELU2>), dim3(N / BN, E), dim3(WAVES * 64), 0, s,
+                       y, x, gather, w, counts, offsets, N, K, N);
   } else {
     DLLM_HOST_CHECK(N % BN == 0, "moe grouped: N must be a multiple of the column tile");
     hipLaunchKernelGGL((moe_grouped_kernel<MTMAX, NT, WAVES, MOE_EPI_STORE>), dim3(N / BN, E), dim3(WAVES * 64), 0, s,
@@ -320,7 +328,7 @@ static void launch_grouped(hipStream_t s, bf16* y, const bf16* x, const int* gat
   }
 }
 
-// mode 1 (SwiGLU): w [E, 2I, K] -> y [T*k, I]; mode 0: w [E, N, K] -> y [T*k, N].
+// mode 1 (SwiGLU): w [E, 2I, K] -> y [T*k, I]; mode 0: w [E, N, K] -> y [T*k, N]; mode 2: as 0, storing max(v, 0)^2.
 // rows_hint = expected rows per expert (T*k/E) picks the kernel family; variant > 0 forces one
 // (benchmarking: 1 = <1,4,8>, 2 = <2,4,8>, 3 = <4,2,8>, 4 = <2,4,4>, 5 = <4,4,4>, 6 = <2,2,8>).
 void moe_grouped_gemm(uintptr_t y, uintptr_t x, uintptr_t gather, uintptr_t w, uintptr_t counts, uintptr_t offsets,
@@ -355,6 +363,185 @@ void moe_combine(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t i
   if (T == 0) return;
   hipLaunchKernelGGL(moe_combine_kernel, dim3(T), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), (bf16*)out,
                      (const bf16*)ysorted, (const float*)topk_w, (const int*)inv, H, k);
+  DLLM_HIP_CHECK(hipGetLastError());
+}
+
+// ------------------------------------------------------------------ grouped-choice router
+// s = sigmoid(logit) (float32 logits [T, ld], the first E columns).  SELECTION ranks s + correction[e]:
+// the experts are split into `groups` contiguous blocks of equal size, blocks are ranked by the sum of
+// their top two selection values, experts outside the `keep` highest-ranked blocks are masked with -inf,
+// and the k highest remaining values are selected.  The mixing WEIGHTS are the selected experts' plain
+// s, normalised to sum one (+ 1e-20 in the divisor) and multiplied by `scale`.  One thread per token, 128 tokens per
+// workgroup; moe_scatter_wide_kernel (one workgroup, LDS counters) then makes the counts / offsets /
+// expert-sorted slot lists that the grouped GEMMs and the combine read.
+constexpr int kMaxGroups = 64;
+constexpr int kMaxChoiceExperts = 256;
+
+template <int EMAX>
+__global__ void __launch_bounds__(128) moe_choice_groups_kernel(
+    const float* __restrict__ logits, long ld, const float* __restrict__ correction, int T, int E, int k, int groups,
+    int keep, float scale, float* __restrict__ topk_w, int* __restrict__ topk_ids) {
+  const int t = blockIdx.x * 128 + threadIdx.x;
+  if (t >= T) return;
+  const int gsz = E / groups;
+  float sc[EMAX], ch[EMAX];
+  for (int e = 0; e < E; ++e) {
+    sc[e] = 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e]));
+    ch[e] = sc[e] + (correction ? correction[e] : 0.f);
+  }
+  if (keep < groups) {
+    float gs[kMaxGroups];
+    for (int g = 0; g < groups; ++g) {
+      float a = -INFINITY, b = -INFINITY;          // top two of the block
+      for (int e = g * gsz; e < (g + 1) * gsz; ++e) {
+        if (ch[e] > a) { b = a; a = ch[e]; }
+        else if (ch[e] > b) b = ch[e];
+      }
+      gs[g] = gsz > 1 ? a + b : a;
+    }
+    unsigned long long kept = 0ull;
+    for (int j = 0; j < keep; ++j) {
+      int best = -1;
+      float bv = -INFINITY;
+      for (int g = 0; g < groups; ++g)
+        if (!((kept >> g) & 1ull) && (best < 0 || gs[g] > bv)) { bv = gs[g]; best = g; }
+      kept |= 1ull << best;
+    }
+    for (int g = 0; g < groups; ++g)
+      if (!((kept >> g) & 1ull))
+        for (int e = g * gsz; e < (g + 1) * gsz; ++e) ch[e] = -INFINITY;
+  }
+  int ids[16];
+  float tot = 0.f;
+  for (int j = 0; j < k; ++j) {
+    int best = -1;
+    float bv = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+      bool taken = false;
+      for (int i = 0; i < j; ++i) taken = taken || ids[i] == e;
+      if (!taken && (best < 0 || ch[e] > bv)) { bv = ch[e]; best = e; }
+    }
+    ids[j] = best;
+    tot += sc[best];
+  }
+  for (int j = 0; j < k; ++j) {
+    topk_ids[t * k + j] = ids[j];
+    topk_w[t * k + j] = sc[ids[j]] / (tot + 1e-20f) * scale;
+  }
+}
+
+__global__ void __launch_bounds__(1024) moe_scatter_wide_kernel(const int* __restrict__ topk_ids, int T, int E, int k,
+                                                                int* __restrict__ counts, int* __restrict__ offsets,
+                                                                int* __restrict__ sorted_tok, int* __restrict__ inv) {
+  __shared__ int cnt[kMaxChoiceExperts], cur[kMaxChoiceExperts];
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int i = threadIdx.x; i < T * k; i += blockDim.x) atomicAdd(&cnt[topk_ids[i]], 1);
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int acc = 0;
+    for (int e = 0; e < E; ++e) {
+      offsets[e] = acc;
+      cur[e] = acc;
+      counts[e] = cnt[e];
+      acc += cnt[e];
+    }
+    offsets[E] = acc;
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < T * k; i += blockDim.x) {
+    const int slot = atomicAdd(&cur[topk_ids[i]], 1);
+    sorted_tok[slot] = i / k;
+    inv[i] = slot;
+  }
+}
+
+void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, int E, int k, int groups, int keep,
+                      float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts, uintptr_t offsets,
+                      uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream) {
+  DLLM_HOST_CHECK(E >= 1 && E <= kMaxChoiceExperts && ld >= E, "1 <= experts <= 256");
+  DLLM_HOST_CHECK(k >= 1 && k <= 16 && k <= E, "1 <= top <= min(16, experts)");
+  DLLM_HOST_CHECK(groups >= 1 && groups <= kMaxGroups && E % groups == 0 && keep >= 1 && keep <= groups &&
+                      keep * (E / groups) >= k,
+                  "expert groups");
+  if (T <= 0) return;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define ROUTE_G(EMAX)                                                                                              \
+  hipLaunchKernelGGL(moe_choice_groups_kernel<EMAX>, dim3((T + 127) / 128), dim3(128), 0, s, (const float*)logits, \
+                     ld, (const float*)correction, T, E, k, groups, keep, scale, (float*)topk_w, (int*)topk_ids)
+  if (E <= 16) ROUTE_G(16);
+  else if (E <= 64) ROUTE_G(64);
+  else ROUTE_G(256);
+#undef ROUTE_G
+  DLLM_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL(moe_scatter_wide_kernel, dim3(1), dim3(1024), 0, s, (const int*)topk_ids, T, E, k, (int*)counts,
+                     (int*)offsets, (int*)sorted_tok, (int*)inv);
+  DLLM_HIP_CHECK(hipGetLastError());
+}
+
+// y <- max(y, 0)^2 in place (activation of experts of the form down(act(up x)))
+template <typename T>
+__global__ void __launch_bounds__(256) relu_sq_kernel(T* __restrict__ y, long n) {
+  for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < n; i += (long)gridDim.x * 256) {
+    const float v = fmaxf((float)y[i], 0.f);
+    y[i] = (T)(v * v);
+  }
+}
+
+void relu_sq(uintptr_t y, long n, int f32, uintptr_t stream) {
+  if (n <= 0) return;
+  const int grid = (int)std::min<long>((n + 255) / 256, 256L * 32);
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  if (f32) hipLaunchKernelGGL(relu_sq_kernel<float>, dim3(grid), dim3(256), 0, s, (float*)y, n);
+  else hipLaunchKernelGGL(relu_sq_kernel<bf16>, dim3(grid), dim3(256), 0, s, (bf16*)y, n);
+  DLLM_HIP_CHECK(hipGetLastError());
+}
+
+// out[t] = sum_j w[t, j] y[inv[t, j]]  (+ sigmoid(gate_logits[t * gate_ld]) * shared[t]: an expert that
+// every token uses, scaled by one gate per token); T = bf16 or float, V elements per lane and step
+template <typename T, int V>
+__global__ void __launch_bounds__(256) moe_combine_gated_kernel(T* __restrict__ out, const T* __restrict__ ysorted,
+                                                                const float* __restrict__ topk_w,
+                                                                const int* __restrict__ inv,
+                                                                const T* __restrict__ shared,
+                                                                const float* __restrict__ gate_logits, long gate_ld,
+                                                                int H, int k) {
+  const int t = blockIdx.x;
+  float gate = 1.f;
+  if (shared && gate_logits) gate = 1.0f / (1.0f + expf(-gate_logits[(size_t)t * gate_ld]));
+  for (int i = threadIdx.x * V; i < H; i += 256 * V) {
+    float acc[V];
+#pragma unroll
+    for (int e = 0; e < V; ++e) acc[e] = 0.f;
+    for (int j = 0; j < k; ++j) {
+      const float wj = topk_w[t * k + j];
+      float y[V];
+      ldv<V>(ysorted + (size_t)inv[t * k + j] * H + i, y);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += wj * y[e];
+    }
+    if (shared) {
+      float y[V];
+      ldv<V>(shared + (size_t)t * H + i, y);
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] += gate * y[e];
+    }
+    stv<V>(out + (size_t)t * H + i, acc);
+  }
+}
+
+void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,
+                       uintptr_t gate_logits, long gate_ld, int T, int H, int k, int f32, uintptr_t stream) {
+  if (T == 0) return;
+  DLLM_HOST_CHECK(H > 0 && k >= 1 && out && ysorted && topk_w && inv, "moe combine arguments");
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define COMBINE_G(TY, V)                                                                                          \
+  hipLaunchKernelGGL((moe_combine_gated_kernel<TY, V>), dim3(T), dim3(256), 0, s, (TY*)out, (const TY*)ysorted,   \
+                     (const float*)topk_w, (const int*)inv, (const TY*)shared, (const float*)gate_logits, gate_ld, \
+                     H, k)
+  if (f32) { if (H % 8 == 0) COMBINE_G(float, 8); else COMBINE_G(float, 1); }
+  else { if (H % 8 == 0) COMBINE_G(bf16, 8); else COMBINE_G(bf16, 1); }
+#undef COMBINE_G
   DLLM_HIP_CHECK(hipGetLastError());
 }
 

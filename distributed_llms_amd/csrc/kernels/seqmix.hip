@@ -12,75 +12,9 @@
 
 #include "common.h"
 #include "launchers.h"
+#include "stream_common.h"
 
 namespace dllm {
-
-template <typename T> __device__ __forceinline__ float ldf(const T* p) { return (float)*p; }
-template <typename T> __device__ __forceinline__ void stf(T* p, float v) { *p = (T)v; }
-
-// V consecutive elements <-> float registers: V = 8 moves 16 bytes of bf16 (32 of float) per lane and
-// needs the address aligned to 8 elements; V = 1 is the any-size form.
-template <int V> __device__ __forceinline__ void ldv(const bf16* p, float (&o)[V]) {
-  if constexpr (V == 2) {
-    const bf16x2 v = *reinterpret_cast<const bf16x2*>(p);
-    o[0] = bf2f(v[0]), o[1] = bf2f(v[1]);
-  } else if constexpr (V == 8) {
-    const bf16x8 v = *reinterpret_cast<const bf16x8*>(p);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) o[j] = bf2f(v[j]);
-  } else {
-#pragma unroll
-    for (int j = 0; j < V; ++j) o[j] = bf2f(p[j]);
-  }
-}
-template <int V> __device__ __forceinline__ void ldv(const float* p, float (&o)[V]) {
-  if constexpr (V == 2) {
-    const f32x2 v = *reinterpret_cast<const f32x2*>(p);
-    o[0] = v[0], o[1] = v[1];
-  } else if constexpr (V == 8) {
-    const f32x4 a = *reinterpret_cast<const f32x4*>(p), b = *reinterpret_cast<const f32x4*>(p + 4);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) o[j] = a[j], o[4 + j] = b[j];
-  } else {
-#pragma unroll
-    for (int j = 0; j < V; ++j) o[j] = p[j];
-  }
-}
-template <int V> __device__ __forceinline__ void stv(bf16* p, const float (&o)[V]) {
-  if constexpr (V == 2) {
-    bf16x2 v;
-    v[0] = f2bf(o[0]), v[1] = f2bf(o[1]);
-    *reinterpret_cast<bf16x2*>(p) = v;
-  } else if constexpr (V == 8) {
-    bf16x8 v;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) v[j] = f2bf(o[j]);
-    *reinterpret_cast<bf16x8*>(p) = v;
-  } else {
-#pragma unroll
-    for (int j = 0; j < V; ++j) p[j] = f2bf(o[j]);
-  }
-}
-template <int V> __device__ __forceinline__ void stv(float* p, const float (&o)[V]) {
-  if constexpr (V == 2) {
-    *reinterpret_cast<f32x2*>(p) = f32x2{o[0], o[1]};
-  } else if constexpr (V == 8) {
-    *reinterpret_cast<f32x4*>(p) = f32x4{o[0], o[1], o[2], o[3]};
-    *reinterpret_cast<f32x4*>(p + 4) = f32x4{o[4], o[5], o[6], o[7]};
-  } else {
-#pragma unroll
-    for (int j = 0; j < V; ++j) p[j] = o[j];
-  }
-}
-
-#define SM_DISPATCH(f32, KERNEL, grid, block, lds, stream, ...)                                        \
-  do {                                                                                                 \
-    if (f32)                                                                                           \
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<float>), grid, block, lds, (hipStream_t)(stream), __VA_ARGS__); \
-    else                                                                                               \
-      hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<bf16>), grid, block, lds, (hipStream_t)(stream), __VA_ARGS__);  \
-    DLLM_HIP_CHECK(hipGetLastError());                                                                 \
-  } while (0)
 
 // --------------------------------------------------------------------------- embedding -> f32
 template <typename T>
@@ -131,19 +65,6 @@ __global__ void __launch_bounds__(256) sm_rms_norm_kernel(void* __restrict__ y_,
   }
 }
 
-#define SM_DISPATCH_V(f32, vec, KERNEL, grid, block, lds, stream, ...)                                          \
-  do {                                                                                                          \
-    hipStream_t s_ = (hipStream_t)(stream);                                                                     \
-    if (f32) {                                                                                                  \
-      if (vec) hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<float, 8>), grid, block, lds, s_, __VA_ARGS__);        \
-      else hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<float, 1>), grid, block, lds, s_, __VA_ARGS__);            \
-    } else {                                                                                                    \
-      if (vec) hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<bf16, 8>), grid, block, lds, s_, __VA_ARGS__);         \
-      else hipLaunchKernelGGL(HIP_KERNEL_NAME(KERNEL<bf16, 1>), grid, block, lds, s_, __VA_ARGS__);             \
-    }                                                                                                           \
-    DLLM_HIP_CHECK(hipGetLastError());                                                                          \
-  } while (0)
-
 void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, float eps, float offset, int f32,
                  uintptr_t stream) {
   if (rows <= 0) return;
@@ -153,13 +74,14 @@ void sm_rms_norm(uintptr_t y, uintptr_t x, uintptr_t w, int rows, int width, flo
 }
 
 // --------------------------------------------------------------------------- close of a sublayer
-// x += mult * rms_norm(o + bias) * (1 + w_post);  h = rms_norm(x) * (1 + w_next) when w_next.
+// x += mult * rms_norm(o + bias) * (offset + w_post);  h = rms_norm(x) * (offset + w_next) when w_next
+// (offset 1: weights stored around zero; 0: plain weights).
 template <typename T, int V>
 __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict__ x, const void* __restrict__ o_,
                                                                const void* __restrict__ bias_,
                                                                const void* __restrict__ wp_,
                                                                const void* __restrict__ wn_, void* __restrict__ h_,
-                                                               int width, float eps, float mult) {
+                                                               int width, float eps, float mult, float offset) {
   __shared__ float red[16];
   const T* o = (const T*)o_ + (size_t)blockIdx.x * width;
   const T* bias = (const T*)bias_;
@@ -193,7 +115,7 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
     ldv<V>(xr + i, xv);
 #pragma unroll
     for (int j = 0; j < V; ++j) {
-      xv[j] = xv[j] + mult * (v[j] * inv * (1.0f + g[j]));
+      xv[j] = xv[j] + mult * (v[j] * inv * (offset + g[j]));
       s2 += xv[j] * xv[j];
     }
     stv<V>(xr + i, xv);
@@ -207,17 +129,17 @@ __global__ void __launch_bounds__(256) sm_post_norm_add_kernel(float* __restrict
     ldv<V>(xr + i, xv);
     ldv<V>(wn + i, g);
 #pragma unroll
-    for (int j = 0; j < V; ++j) xv[j] = xv[j] * inv2 * (1.0f + g[j]);
+    for (int j = 0; j < V; ++j) xv[j] = xv[j] * inv2 * (offset + g[j]);
     stv<V>(h + i, xv);
   }
 }
 
 void sm_post_norm_add(uintptr_t x, uintptr_t o, uintptr_t bias, uintptr_t w_post, uintptr_t w_next, uintptr_t h,
-                      int rows, int width, float eps, float mult, int f32, uintptr_t stream) {
+                      int rows, int width, float eps, float mult, float offset, int f32, uintptr_t stream) {
   if (rows <= 0) return;
   DLLM_HOST_CHECK(width > 0 && (!w_next || h), "post_norm_add arguments");
   SM_DISPATCH_V(f32, width % 8 == 0, sm_post_norm_add_kernel, dim3(rows), dim3(256), 0, stream, (float*)x,
-                (const void*)o, (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult);
+                (const void*)o, (const void*)bias, (const void*)w_post, (const void*)w_next, (void*)h, width, eps, mult, offset);
 }
 
 // --------------------------------------------------------------------------- causal convolution with state

@@ -223,8 +223,11 @@ def build_decode_batch(seq_ids: np.ndarray, seq_lens: np.ndarray, bm, block_size
                                  int(seq_lens.max()) if b else 0, slot, step_id, None), seq_ids, bm)
 
 
-def to_device_meta(hb: HostBatch, device, pad_ctx_to: Optional[int] = None) -> (torch.Tensor, BatchMeta):
-    """Upload a HostBatch; returns (ids tensor, BatchMeta)."""
+def to_device_meta(hb: HostBatch, device, pad_ctx_to: Optional[int] = None,
+                   seq_index: bool = False) -> (torch.Tensor, BatchMeta):
+    """Upload a HostBatch; returns (ids tensor, BatchMeta).  ``seq_index``: also each token's sequence
+    index and the chunk offsets in decode steps (models whose kernels take varlen metadata in every
+    step); batches that carry state slots get them anyway."""
     dev = torch.device(device)
     nb = dev.type == "cuda"
     def up(a, dtype=torch.int32):
@@ -242,6 +245,7 @@ def to_device_meta(hb: HostBatch, device, pad_ctx_to: Optional[int] = None) -> (
         num_tokens=hb.num_tokens)
     if hb.state_slots is not None:
         meta.state_slots = up(hb.state_slots)
+    if hb.state_slots is not None or seq_index:
         meta.tok_seq = up(np.repeat(np.arange(hb.num_seqs, dtype=np.int32), np.diff(hb.cu_seqlens)))
         if meta.cu_seqlens_q is None:
             meta.cu_seqlens_q = up(hb.cu_seqlens)

@@ -49,7 +49,8 @@ class DecodeGraphRunner:
         # models with per-sequence state: a decode step is one token per sequence, so the token ->
         # sequence map and the chunk offsets are constants
         self.with_state = bool(getattr(cfg, "needs_state_slots", False))
-        self.row_ids = torch.arange(mb + 1, dtype=torch.int32, device=dev) if self.with_state else None
+        self.with_seq_index = self.with_state or bool(getattr(cfg, "needs_seq_index", False))
+        self.row_ids = torch.arange(mb + 1, dtype=torch.int32, device=dev) if self.with_seq_index else None
         self.hidden = None if stage.is_first else torch.zeros(mb, stage.in_width, dtype=stage.dtype, device=dev)
         max_splits = 64
         self.ws = (torch.empty(mb * cfg.num_heads * max_splits * cfg.head_dim, dtype=torch.float32, device=dev),
@@ -75,6 +76,7 @@ class DecodeGraphRunner:
                          max_ctx=cb, num_seqs=bb, num_tokens=bb, attn_workspace=self.ws)
         if self.with_state:
             meta.state_slots = self.state_slots[:bb]
+        if self.with_seq_index:
             meta.tok_seq = self.row_ids[:bb]
             meta.cu_seqlens_q = self.row_ids[:bb + 1]
         return meta

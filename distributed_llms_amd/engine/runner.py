@@ -73,7 +73,7 @@ class StageRunner:
         self.max_blocks = -(-ecfg.max_seq_len // self.block_size)
         self._busy = None                 # [(start, end) events or host seconds] while metering
         self.graph_sets = []
-        if ecfg.use_graphs and stage.device.type == "cuda":
+        if ecfg.use_graphs and stage.device.type == "cuda" and getattr(stage, "graph_capturable", True):
             sizes = [b for b in ecfg.graph_batch_sizes if b <= ecfg.max_batch] or [ecfg.max_batch]
             if max(sizes) < ecfg.max_batch:
                 sizes.append(ecfg.max_batch)
@@ -106,7 +106,7 @@ class StageRunner:
         gr = self.graph_sets[slot % len(self.graph_sets)] if self.graph_sets else None
         if (not hb.is_prefill) and gr is not None and gr.can_run(hb.num_seqs, hb.max_ctx):
             return gr.run(hb, hidden, ids_dev=ids_dev)
-        ids, meta = to_device_meta(hb, st.device)
+        ids, meta = to_device_meta(hb, st.device, seq_index=getattr(st.cfg, "needs_seq_index", False))
         if ids_dev is not None:
             ids = ids_dev.to(torch.int32)
         return st.forward(ids if st.is_first else hidden, meta)

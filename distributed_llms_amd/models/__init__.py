@@ -5,6 +5,9 @@ def stage_class(arch: str):
     if arch == "tudilix":
         from .hybrid import HybridStage
         return HybridStage
+    if arch == "gikovik":
+        from .gikovik import GikovikStage
+        return GikovikStage
     if arch in ("llama", "mixtral", "gpt2"):
         from .stage import ModelStage
         return ModelStage

@@ -106,14 +106,20 @@ def synth_state_dict(cfg: ModelConfig, seed: int = 0, dtype=torch.float32) -> Di
     return sd
 
 
-class HybridStage:
-    """All layers of a layer-list model on one device (see the module docstring)."""
+class LayerListStage:
+    """What the stages of layer-list models share: one stage owns every layer of the ``config.json`` list
+    on one device (no pipeline cuts, no tensor parallelism), a float32 residual stream, per-cache paged
+    K/V tensors of their own shapes behind ONE block table (the engine's BlockManager), and the same
+    interface as :class:`~.stage.ModelStage` (``forward(ids, BatchMeta)``, ``allocate_kv``,
+    ``load_hf_state``, ``init_synthetic``), so the engine, scheduler and sampler drive them unchanged.
+    A subclass gives ``cache_shapes`` (per cache key the K and V shapes inside a block), the weights
+    and ``forward``."""
 
     def __init__(self, cfg: ModelConfig, layer_start: int = 0, layer_end: Optional[int] = None, device="cpu",
                  dtype=torch.bfloat16, units: Optional[tuple] = None, tp=None, unit_group: int = 2):
         from ..parallel.tensor_parallel import TPGroup
         if cfg.layers is None:
-            raise ValueError("HybridStage needs a layer-list config")
+            raise ValueError(f"{type(self).__name__} needs a layer-list config")
         layer_end = cfg.num_layers if layer_end is None else layer_end
         if (layer_start, layer_end) != (0, cfg.num_layers) or (units is not None and tuple(units) != (
                 0, unit_group * cfg.num_layers)):
@@ -130,6 +136,80 @@ class HybridStage:
         self.is_first = self.is_last = True
         self.specs = cfg.layers
         self.hkv = cfg.num_kv_heads
+        self.layers: List[Dict[str, torch.Tensor]] = []
+        self.embed: Dict[str, torch.Tensor] = {}
+        self.head: Dict[str, torch.Tensor] = {}
+        self.kv = None                 # _PagedCaches: {cache key: (k_cache, v_cache)} + block_size / num_blocks
+        self.state = None
+        self.num_state_slots = 0
+        self.taps = None               # optional list: the residual stream after every layer run (debugging)
+
+    # ------------------------------------------------------------------ what a subclass provides
+    def cache_shapes(self, block_size: int) -> Dict[Any, tuple]:
+        """{cache key: (k shape, v shape)} of one block (without the leading block axis)."""
+        raise NotImplementedError
+
+    def quantize(self, mode):
+        if mode not in ("", "none", None):
+            raise ValueError("layer-list models run unquantized")
+        return self
+
+    def weight_bytes(self) -> int:
+        def walk(o):
+            if isinstance(o, torch.Tensor):
+                return o.numel() * o.element_size()
+            if isinstance(o, dict):
+                return sum(walk(v) for v in o.values())
+            return 0
+        return sum(walk(d) for d in self.layers) + walk(self.embed) + walk(self.head)
+
+    def lm_head_weight(self, full: bool = False) -> torch.Tensor:
+        return self.head["lm_head"]
+
+    def needs_embed(self) -> bool:
+        return True
+
+    @property
+    def num_layers(self) -> int:
+        """Caches that take a share of every block (what the K/V pool is planned for)."""
+        return len(self.cache_shapes(1))
+
+    # ------------------------------------------------------------------ cache
+    def kv_bytes_per_block(self, block_size: int) -> int:
+        e = torch.empty((), dtype=self.dtype).element_size()
+        n = sum(torch.Size(k).numel() + torch.Size(v).numel() for k, v in self.cache_shapes(block_size).values())
+        return max(1, n * e)
+
+    def allocate_kv(self, num_blocks: int, block_size: int):
+        caches = {key: (torch.zeros(num_blocks, *ks, dtype=self.dtype, device=self.device),
+                        torch.zeros(num_blocks, *vs, dtype=self.dtype, device=self.device))
+                  for key, (ks, vs) in self.cache_shapes(block_size).items()}
+        self.kv = _PagedCaches(caches, num_blocks, block_size)
+        return self.kv
+
+    def _seq_batch(self, meta: BatchMeta) -> sm.SeqBatch:
+        if meta.tok_seq is None or meta.cu_seqlens_q is None or (
+                self.cfg.needs_state_slots and meta.state_slots is None):
+            raise RuntimeError("a layer-list model needs varlen metadata in every step (and, with per-sequence "
+                               "state, a BlockManager with num_state_slots > 0)")
+        return sm.SeqBatch(meta.cu_seqlens_q, meta.positions, meta.tok_seq, meta.state_slots, meta.num_seqs,
+                           meta.num_tokens, max(1, meta.max_q_len))
+
+
+class HybridStage(LayerListStage):
+    """All layers of a Tudilix model on one device (see the module docstring)."""
+
+    @staticmethod
+    def layer_param_count(width: int, layer: Dict[str, Any]) -> int:
+        return layer_param_count(width, layer)
+
+    @staticmethod
+    def kv_elements_per_token(cfg: ModelConfig) -> int:
+        return sum(kv_width(l) for l in cfg.layers)
+
+    def __init__(self, cfg: ModelConfig, layer_start: int = 0, layer_end: Optional[int] = None, device="cpu",
+                 dtype=torch.bfloat16, units: Optional[tuple] = None, tp=None, unit_group: int = 2):
+        super().__init__(cfg, layer_start, layer_end, device, dtype, units, tp, unit_group)
         for i, layer in enumerate(self.specs):
             m = layer["mixer"]
             if layer["type"] == "attention":
@@ -145,25 +225,15 @@ class HybridStage:
             elif m["width"] % m["blocks"]:
                 raise ValueError(f"layer {i}: width is not a multiple of blocks")
         self.kv_layers = [i for i, l in enumerate(self.specs) if kv_width(l)]
-        self.layers: List[Dict[str, torch.Tensor]] = []
-        self.embed: Dict[str, torch.Tensor] = {}
-        self.head: Dict[str, torch.Tensor] = {}
-        self.kv = None                 # {layer: (k_cache, v_cache)} + block_size / num_blocks
         self.state = None              # per layer {"conv": ..., "s": ...}
-        self.num_state_slots = 0
         self.rot = {}                  # layer -> (freqs [dims/2] f32, magnitude)
         for i, l in enumerate(self.specs):
             if l["type"] == "attention":
                 r = l["mixer"]["rot"]
                 f, mag = sm.yarn_frequencies(r["dims"], r["base"], r.get("scaling"))
                 self.rot[i] = (f.to(self.device), mag)
-        self.taps = None               # optional list: the residual stream after every layer (debugging)
 
     # ------------------------------------------------------------------ weights
-    @property
-    def num_layers(self) -> int:
-        return len(self.kv_layers)
-
     def load_hf_state(self, sd: Dict[str, torch.Tensor]) -> "HybridStage":
         """From checkpoint-named tensors: fuses y|x, q|k|v (and their convolutions), gate|up, and stores
         the gate matrices transposed ([blocks, in, out]) and the convolution weights tap-major ([taps, C])."""
@@ -208,36 +278,15 @@ class HybridStage:
     def init_synthetic(self, seed: int = 0) -> "HybridStage":
         return self.load_hf_state(synth_state_dict(self.cfg, seed))
 
-    def quantize(self, mode) -> "HybridStage":
-        if mode not in ("", "none", None):
-            raise ValueError("layer-list models run unquantized")
-        return self
-
-    def weight_bytes(self) -> int:
-        n = sum(t.numel() * t.element_size() for d in self.layers for t in d.values())
-        return n + sum(t.numel() * t.element_size() for d in (self.embed, self.head) for t in d.values())
-
-    def lm_head_weight(self, full: bool = False) -> torch.Tensor:
-        return self.head["lm_head"]
-
-    def needs_embed(self) -> bool:
-        return True
-
     # ------------------------------------------------------------------ cache and state
-    def kv_bytes_per_block(self, block_size: int) -> int:
-        e = torch.empty((), dtype=self.dtype).element_size()
-        return max(1, sum(kv_width(l) for l in self.specs) * block_size * e)
-
-    def allocate_kv(self, num_blocks: int, block_size: int):
+    def cache_shapes(self, block_size: int) -> Dict[Any, tuple]:
         """Paged caches of the attention layers with K/V of their own: k [NB, G, BS, dim],
         v [NB, G, vdim, BS] (transposed inside a block); a ``kv_from`` layer reads its source's pair."""
-        caches = {}
+        out = {}
         for i in self.kv_layers:
             m = self.specs[i]["mixer"]
-            caches[i] = (torch.zeros(num_blocks, m["kv_heads"], block_size, m["dim"], dtype=self.dtype, device=self.device),
-                         torch.zeros(num_blocks, m["kv_heads"], m["vdim"], block_size, dtype=self.dtype, device=self.device))
-        self.kv = _PagedCaches(caches, num_blocks, block_size)
-        return self.kv
+            out[i] = ((m["kv_heads"], block_size, m["dim"]), (m["kv_heads"], m["vdim"], block_size))
+        return out
 
     def allocate_state(self, num_slots: int):
         """State pools, one row per BlockManager state slot: per layer the convolution tail
@@ -270,13 +319,6 @@ class HybridStage:
         return n
 
     # ------------------------------------------------------------------ forward
-    def _seq_batch(self, meta: BatchMeta) -> sm.SeqBatch:
-        if meta.state_slots is None or meta.tok_seq is None or meta.cu_seqlens_q is None:
-            raise RuntimeError("a layer-list model needs state slots in the batch metadata "
-                               "(a BlockManager with num_state_slots > 0)")
-        return sm.SeqBatch(meta.cu_seqlens_q, meta.positions, meta.tok_seq, meta.state_slots, meta.num_seqs,
-                           meta.num_tokens, max(1, meta.max_q_len))
-
     def _attention(self, i: int, h: torch.Tensor, w, meta: BatchMeta, sb: sm.SeqBatch) -> torch.Tensor:
         m = self.specs[i]["mixer"]
         own = "kv_from" not in m

@@ -15,6 +15,7 @@ CPU path: the PyTorch reference (ops/reference.py).
 """
 from __future__ import annotations
 
+from typing import Optional
 
 import torch
 import torch.nn.functional as F
@@ -140,4 +141,113 @@ def forward(x: torch.Tensor, w_router: torch.Tensor, w_gate_up: torch.Tensor, w_
                 ys[a:b] = F.linear(linear_swiglu(xs[a:b], w_gate_up[j]), w_down[j])
     out = torch.empty_like(x)
     k.moe_combine(out.data_ptr(), ys.data_ptr(), topk_w.data_ptr(), inv.data_ptr(), t, h, top_k, st)
+    return out
+
+
+# ------------------------------------------------------------------ grouped-choice router, squared-ReLU experts
+def route_grouped_choice(logits: torch.Tensor, correction: Optional[torch.Tensor], num_experts: int, top: int,
+                         groups: int = 1, keep: int = 1, scale: float = 1.0):
+    """Reference (PyTorch, any device) of the grouped-choice router: scores s = sigmoid(logits[:, :E]);
+    selection ranks s + correction; the experts are split into ``groups`` contiguous blocks of equal size,
+    blocks are ranked by the sum of their top two selection values, and experts outside the ``keep``
+    highest-ranked blocks are masked with -inf; the mixing weights are the selected experts' plain s,
+    normalised to sum one (+ 1e-20 in the divisor) and multiplied by ``scale``.  Returns (weights
+    [T, top] float32, ids [T, top] int64)."""
+    t = logits.shape[0]
+    e = num_experts
+    s = torch.sigmoid(logits[:, :e].float())
+    ch = s if correction is None else s + correction.float()
+    if keep < groups:
+        gsz = e // groups
+        gs = ch.view(t, groups, gsz).topk(min(2, gsz), dim=-1).values.sum(-1)
+        kept = torch.zeros(t, groups, dtype=torch.bool, device=logits.device)
+        kept.scatter_(1, gs.topk(keep, dim=-1).indices, True)
+        ch = ch.masked_fill(~kept.repeat_interleave(gsz, 1), float("-inf"))
+    ids = ch.topk(top, dim=-1).indices
+    w = s.gather(1, ids)
+    return w / (w.sum(-1, keepdim=True) + 1e-20) * scale, ids
+
+
+def grouped_choice_ffn(x: torch.Tensor, w_router: torch.Tensor, correction: Optional[torch.Tensor],
+                       w_up: torch.Tensor, w_down: torch.Tensor, top: int, groups: int = 1, keep: int = 1,
+                       scale: float = 1.0, shared_up: Optional[torch.Tensor] = None,
+                       shared_down: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Mixture of experts of the form down_e(relu(up_e x)^2) with the grouped-choice router
+    (:func:`route_grouped_choice`).  ``w_router`` [E (+ 1), W] float32: the router rows, then -- with a
+    shared expert -- the row of its gate; the logits are a float32 product.  ``w_up`` [E, F, W],
+    ``w_down`` [E, W, F].  ``shared_up`` [Fs, W] / ``shared_down`` [W, Fs]: an expert of the same form that
+    every token uses, times sigmoid(gate logit), one gate per token."""
+    e, f, width = w_up.shape
+    t = x.shape[0]
+    has_shared = shared_up is not None
+    if w_router.shape[0] != e + (1 if has_shared else 0) or w_router.dtype != torch.float32:
+        raise ValueError("grouped_choice_ffn: router rows = experts (+ 1 with a shared expert), float32")
+    logits = F.linear(x.float(), w_router)                       # float32 also for bf16 activations
+    if not x.is_cuda:
+        tw, ids = route_grouped_choice(logits, correction, e, top, groups, keep, scale)
+        out = torch.zeros(t, width, dtype=torch.float32)
+        xf = x.float()
+        for j in range(e):
+            rows, col = (ids == j).nonzero(as_tuple=True)
+            if rows.numel():
+                y = F.linear(torch.relu(F.linear(xf[rows], w_up[j].float())).square(), w_down[j].float())
+                out.index_add_(0, rows, y * tw[rows, col, None])
+        if has_shared:
+            y = F.linear(torch.relu(F.linear(xf, shared_up.float())).square(), shared_down.float())
+            out += y * torch.sigmoid(logits[:, e:e + 1])
+        return out.to(x.dtype)
+    from . import linear
+    k = _ext.kernels()
+    st = torch.cuda.current_stream().cuda_stream
+    dev = x.device
+    f32 = 1 if x.dtype == torch.float32 else 0
+    if not (x.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous() and logits.is_contiguous()):
+        raise ValueError("grouped_choice_ffn: operands must be contiguous")
+    if correction is not None and (correction.dtype != torch.float32 or correction.numel() != e):
+        raise ValueError("grouped_choice_ffn: correction is float32 [E]")
+    topk_w = torch.empty(t, top, dtype=torch.float32, device=dev)
+    topk_ids = torch.empty(t, top, dtype=torch.int32, device=dev)
+    counts = torch.empty(e, dtype=torch.int32, device=dev)
+    offsets = torch.empty(e + 1, dtype=torch.int32, device=dev)
+    sorted_tok = torch.empty(t * top, dtype=torch.int32, device=dev)
+    inv = torch.empty(t * top, dtype=torch.int32, device=dev)
+    k.moe_route_groups(logits.data_ptr(), logits.shape[1], 0 if correction is None else correction.data_ptr(), t, e,
+                       top, groups, keep, float(scale), topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(),
+                       offsets.data_ptr(), sorted_tok.data_ptr(), inv.data_ptr(), st)
+    slots = t * top
+    ys = torch.empty(slots, width, dtype=x.dtype, device=dev)
+    bf = x.dtype == torch.bfloat16
+    if bf and t <= GROUPED_MAX_TOKENS and width % 128 == 0 and f % 128 == 0:
+        # decode-sized: grouped weight-streaming GEMMs on the expert-sorted slots, no host sync
+        act = torch.empty(slots, f, dtype=x.dtype, device=dev)
+        rows = -(-slots // e)
+        k.moe_grouped_gemm(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_up.data_ptr(), counts.data_ptr(),
+                           offsets.data_ptr(), e, f, width, 2, rows, knobs.K.moe_variant, st)     # mode 2: relu^2
+        k.moe_grouped_gemm(ys.data_ptr(), act.data_ptr(), 0, w_down.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
+                           e, width, f, 0, rows, knobs.K.moe_variant, st)
+    elif bf and f % 256 == 0 and width % 256 == 0 and t * width * 2 < (1 << 32) and slots * f * 2 < (1 << 32):
+        # prompt-sized: one grouped 256 x 256-tile launch per projection over every expert's row tiles
+        act = torch.empty(slots, f, dtype=x.dtype, device=dev)
+        k.gemm_pp_moe(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_up.data_ptr(), counts.data_ptr(),
+                      offsets.data_ptr(), e, f, width, t, slots, 2, st)                                  # mode 2: relu^2
+        k.gemm_pp_moe(ys.data_ptr(), act.data_ptr(), 0, w_down.data_ptr(), counts.data_ptr(), offsets.data_ptr(), e,
+                      width, f, slots, slots, 0, st)
+    else:
+        # float32 and odd expert sizes: per-expert library GEMMs, counts read on the host
+        xs = x.index_select(0, sorted_tok.long())
+        off = offsets.cpu().tolist()
+        for j in range(e):
+            a, b = off[j], off[j + 1]
+            if b > a:
+                u = F.linear(xs[a:b], w_up[j])
+                k.relu_sq(u.data_ptr(), u.numel(), f32, st)
+                ys[a:b] = F.linear(u, w_down[j])
+    sh = None
+    if has_shared:
+        u = linear(x, shared_up)
+        k.relu_sq(u.data_ptr(), u.numel(), f32, st)
+        sh = linear(u, shared_down)
+    out = torch.empty_like(x)
+    k.moe_combine_gated(out.data_ptr(), ys.data_ptr(), topk_w.data_ptr(), inv.data_ptr(), 0 if sh is None else sh.data_ptr(),
+                        logits.data_ptr() + 4 * e if has_shared else 0, logits.shape[1], t, width, top, f32, st)
     return out

@@ -35,7 +35,7 @@ class SeqBatch:
     cu: torch.Tensor            # [B + 1] int32
     positions: torch.Tensor     # [T] int32
     tok_seq: torch.Tensor       # [T] int32
-    state_slots: torch.Tensor   # [B] int32
+    state_slots: Optional[torch.Tensor]   # [B] int32 (None: the model keeps no state besides K/V)
     num_seqs: int
     num_tokens: int
     max_q_len: int
@@ -98,14 +98,16 @@ def rms_norm_f32(x: torch.Tensor, w: torch.Tensor, eps: float, act_dtype, one_pl
 
 
 def post_norm_add(x: torch.Tensor, o: torch.Tensor, w_post: torch.Tensor, eps: float, mult: float,
-                  bias: Optional[torch.Tensor] = None, w_next: Optional[torch.Tensor] = None):
+                  bias: Optional[torch.Tensor] = None, w_next: Optional[torch.Tensor] = None, one_plus: bool = True):
     """The close of a sublayer, fused: ``x += mult * rms_norm(o + bias) * (1 + w_post)`` in place on the
     float32 residual stream; with ``w_next`` also returns the next sublayer's input
-    ``rms_norm(x) * (1 + w_next)`` in ``o``'s dtype (None otherwise)."""
+    ``rms_norm(x) * (1 + w_next)`` in ``o``'s dtype (None otherwise).  ``one_plus`` False: both norm
+    weights are plain (``* w``)."""
+    off = 1.0 if one_plus else 0.0
     if not x.is_cuda:
         ob = o.float() if bias is None else o.float() + bias.float()
-        x.add_(mult * _ref_rms(ob, w_post, eps, 1.0))
-        return x, (None if w_next is None else _ref_rms(x, w_next, eps, 1.0).to(o.dtype))
+        x.add_(mult * _ref_rms(ob, w_post, eps, off))
+        return x, (None if w_next is None else _ref_rms(x, w_next, eps, off).to(o.dtype))
     _ck(x, "x", torch.float32)
     _ck(o, "o")
     t, width = x.shape
@@ -113,7 +115,7 @@ def post_norm_add(x: torch.Tensor, o: torch.Tensor, w_post: torch.Tensor, eps: f
         raise ValueError("post_norm_add: o / x shape mismatch")
     h = torch.empty_like(o) if w_next is not None else None
     _k().sm_post_norm_add(x.data_ptr(), o.data_ptr(), _ptr(bias), w_post.data_ptr(), _ptr(w_next), _ptr(h), t, width,
-                          float(eps), float(mult), _f32flag(o), _stream())
+                          float(eps), float(mult), off, _f32flag(o), _stream())
     return x, h
 
 
@@ -356,14 +358,30 @@ def attn_prep(qkv: torch.Tensor, conv_w: torch.Tensor, state: torch.Tensor, q_no
 
 
 # ------------------------------------------------------------------ sliding-window attention
+DECODE_SPLIT_KEYS = 256     # fewest keys worth a workgroup of their own
+DECODE_TARGET_WGS = 512     # workgroups wanted on the chip (256 CUs, two each)
+
+
+def decode_splits(rows: int, heads: int, kv_heads: int, ctx: int) -> int:
+    """Runs to cut each decode row's keys into: enough workgroups (rows x K/V heads x 16-head groups x
+    runs) to fill the chip, none shorter than DECODE_SPLIT_KEYS keys; 1 when the bound ``ctx`` is unknown."""
+    wgs = max(1, rows * kv_heads * -(-(heads // kv_heads) // 16))
+    return max(1, min(DECODE_TARGET_WGS // wgs, ctx // DECODE_SPLIT_KEYS, 64))
+
+
 def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_tables: torch.Tensor,
-                     sb: SeqBatch, window: int, scale: float, num_decode: Optional[int] = None) -> torch.Tensor:
+                     sb: SeqBatch, window: int, scale: float, num_decode: Optional[int] = None,
+                     sinks: Optional[torch.Tensor] = None, max_ctx: Optional[int] = None) -> torch.Tensor:
     """Softmax attention of every query token over the keys j of its own sequence with
     0 <= p - j < window (p the query's position), keys / values read through ``block_tables`` from
     caches k [NB, G, BS, dim] / v [NB, G, vdim, BS]; query head h reads K/V head h // (H / G).
     Scores and weights are float32.  ``num_decode``: the first that many sequences are one-token
     rows (they take the decode kernel; None: every sequence is one); the rest are prompt chunks.
-    Returns [T, H, vdim]."""
+    ``sinks`` [H] float32: exp(sinks[h]) is added to head h's softmax denominator -- a learned per-head
+    logit that takes part in the normalisation only (nothing is attended to through it; it enters as it
+    is, without the score scale).  ``max_ctx``: a bound on the decode
+    rows' context; with few rows of long context their keys are cut into runs on separate workgroups
+    (results equal up to rounding).  Returns [T, H, vdim]."""
     t, h, d = q.shape
     g, bs, dv = k_cache.shape[1], k_cache.shape[2], v_cache.shape[2]
     if not q.is_cuda:
@@ -378,7 +396,11 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
             kk = k_cache[blk, :, idx % bs].float().repeat_interleave(rep, 1)     # [n, H, d]
             vv = v_cache[blk, :, :, idx % bs].float().repeat_interleave(rep, 1)
             s = torch.einsum("hd,nhd->hn", q[i].float(), kk) * scale
-            out[i] = torch.einsum("hn,nhd->hd", torch.softmax(s, -1), vv)
+            if sinks is not None:      # one more column in the softmax whose weight is dropped
+                p = torch.softmax(torch.cat([s, sinks.float()[:, None]], -1), -1)[:, :-1]
+            else:
+                p = torch.softmax(s, -1)
+            out[i] = torch.einsum("hn,nhd->hd", p, vv)
         return out.to(q.dtype)
     _ck(q, "q")
     _ck(k_cache, "k_cache", q.dtype)
@@ -386,17 +408,25 @@ def window_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tens
     _ck(block_tables, "block_tables", torch.int32)
     if h % g or k_cache.shape[3] != d or v_cache.shape[3] != bs or window < 1:
         raise ValueError("window_attention: head / size mismatch")
+    if sinks is not None:
+        _ck(sinks, "sinks", torch.float32)
+        if sinks.numel() != h:
+            raise ValueError("window_attention: one sink per query head")
     out = torch.empty(t, h, dv, dtype=q.dtype, device=q.device)
     nd = sb.num_seqs if num_decode is None else int(num_decode)
     f = _f32flag(q)
     if nd:       # one-token rows are the first nd tokens
+        splits, ws = decode_splits(nd, h, g, min(int(window), int(max_ctx or 0))), None
+        if splits > 1 and not f:
+            ws = torch.empty(nd * h * splits * (dv + 2), dtype=torch.float32, device=q.device)
         _k().sm_window_attn_decode(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                    block_tables.data_ptr(), block_tables.shape[1], sb.positions.data_ptr(),
-                                   sb.tok_seq.data_ptr(), nd, h, g, d, dv, bs, int(window), float(scale), f, _stream())
+                                   sb.tok_seq.data_ptr(), nd, h, g, d, dv, bs, int(window), float(scale), _ptr(sinks),
+                                   splits if ws is not None else 1, _ptr(ws), f, _stream())
     if t > nd:
         _k().sm_window_attn_prefill(out.data_ptr(), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                     block_tables.data_ptr(), block_tables.shape[1], sb.cu.data_ptr(),
                                     sb.positions.data_ptr(), sb.tok_seq.data_ptr(), nd, sb.num_seqs, t, sb.max_q_len,
                                     h, g, d, dv, bs,
-                                    int(window), float(scale), f, _stream())
+                                    int(window), float(scale), _ptr(sinks), f, _stream())
     return out
