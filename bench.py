@@ -85,10 +85,12 @@ def parse(argv=None):
                     help="record a roctx/host/GPU timeline of the timed steps: DIR/trace_rank<r>.json "
                          "(Chrome format) and per-stage device busy %% in the JSON line")
     ap.add_argument("--hybrid", default=None, metavar="SIZE[,SIZE]",
-                    help="instead of the headline workload: prefill and decode tokens/s of the layer-list hybrid "
-                         "model (Tudilix) beside a Llama-architecture model of equal size (sizes: 2b, 9b, small), "
-                         "--batch prompts of --prompt-len tokens then --gen-len decode steps; one JSON line per size")
-    ap.add_argument("--hybrid-models", default="tudilix,llama", help="--hybrid: which of the two models to run")
+                    help="instead of the headline workload: prefill and decode tokens/s of a layer-list model "
+                         "beside the closest flat-config model of equal size (sizes: 2b, 9b, small), --batch "
+                         "prompts of --prompt-len tokens then --gen-len decode steps; one JSON line per size")
+    ap.add_argument("--hybrid-models", default="tudilix,llama",
+                    help="--hybrid: the models to run: tudilix,llama (sliding-window attention + RG-LRU beside Llama) "
+                         "or gikovik,mixtral (latent attention + grouped-choice experts beside Mixtral), or one of them")
     return ap.parse_args(argv)
 
 

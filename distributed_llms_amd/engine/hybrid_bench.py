@@ -1,6 +1,8 @@
-"""Prefill and decode throughput of the layer-list hybrid model beside a Llama-architecture model of
-equal size (``bench.py --hybrid``): same width, layer count, feed-forward size, head size and K/V
-heads, random weights, one GPU.  Every step goes through the engine's StageRunner (the trace
+"""Prefill and decode throughput of a layer-list model beside the closest flat-config model of equal
+size (``bench.py --hybrid``), random weights, one GPU: Tudilix (sliding-window attention + RG-LRU) beside
+a Llama-architecture model of the same width, layer count, feed-forward size, head size and K/V heads;
+Gikovik (latent attention + grouped-choice mixture of experts) beside a Mixtral-architecture model of the
+same width, layer count, heads, expert count and experts per token, with expert weights of equal size.  Every step goes through the engine's StageRunner (the trace
 replayer builds the batches): one step with ``batch`` prompts of ``prompt_len`` tokens (prefill),
 then ``gen_len`` steps of one token per sequence (decode)."""
 from __future__ import annotations
@@ -47,6 +49,45 @@ def llama_config(size: str, vocab: int = 32000) -> ModelConfig:
                        num_layers=nl, num_heads=h, num_kv_heads=g, head_dim=d, max_position=8192)
 
 
+# name -> (width, layers, dense ff, heads, dim, rot_dim, vdim, kv_rank, q_rank, experts, top, expert ff)
+GIKOVIK_SIZES = {
+    "small": (1024, 6, 3072, 8, 64, 32, 64, 128, 384, 8, 2, 1024),
+    "2b": (2560, 6, 7680, 16, 128, 64, 128, 192, 768, 8, 2, 2560),
+    "9b": (4096, 6, 12288, 32, 128, 64, 128, 192, 1536, 8, 2, 4096),
+}
+
+
+def gikovik_config(size: str, vocab: int = 32000) -> ModelConfig:
+    """Layers 0 and 3 dense, the others mixtures with a shared expert; every third layer the sink form,
+    the others the rotated form; the first three layers as a loop that runs once (its entry projection
+    is part of the step); a 64-column token input."""
+    w, nl, ff, h, d, dr, dv, r, qr, e, top, ef = GIKOVIK_SIZES[size]
+    moe = {"kind": "moe", "expert": {"ff": ef}, "shared": {"ff": ef},
+           "router": {"experts": e, "groups": {"count": 4, "keep": 2}, "scale": 2.5, "top": top}}
+    layers = []
+    for i in range(nl):
+        m = {"heads": h, "dim": d, "vdim": dv, "kv_rank": r + (dr if i % 3 == 2 else 0), "q_rank": qr,
+             "scale": (d + dr) ** -0.5}
+        kind = "latent_attention"
+        if i % 3 != 2:
+            kind = "latent_attention_2"
+            m.update({"rot_dim": dr, "rot": {"base": 10000.0, "dims": dr}})
+        layers.append({"type": kind, "mixer": m, "mlp": {"kind": "dense", "ff": ff} if i % 3 == 0 else moe})
+    return ModelConfig.from_hf_config({"architecture": "Gikovik", "vocab": vocab, "width": w, "norm": {"eps": 1e-6},
+                                       "token_side": {"dim": 64}, "loop": {"start": 0, "stop": 3, "times": 1},
+                                       "layers": layers}, name=f"gikovik-{size}")
+
+
+def mixtral_config(size: str, vocab: int = 32000) -> ModelConfig:
+    """Same width, layers, heads, experts and experts per token; three-matrix SwiGLU experts of 2/3 the
+    width of the two-matrix ones (rounded up to 256), i.e. expert weights of equal size."""
+    w, nl, _ff, h, _d, _dr, _dv, _r, _qr, e, top, ef = GIKOVIK_SIZES[size]
+    inter = -(-(2 * ef // 3) // 256) * 256
+    return ModelConfig(name=f"mixtral-{size}", arch="mixtral", vocab_size=vocab, hidden_size=w, intermediate_size=inter,
+                       num_layers=nl, num_heads=h, num_kv_heads=max(1, h // 4), head_dim=128, max_position=8192,
+                       rope_theta=1000000.0, num_experts=e, experts_per_token=top)
+
+
 def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps: int, tmp: str, graphs: bool):
     import os
     os.makedirs(tmp, exist_ok=True)
@@ -83,18 +124,23 @@ def _measure(mcfg: ModelConfig, batch: int, prompt_len: int, gen_len: int, reps:
     return batch * prompt_len / min(pre), batch * gen_len / min(dec)
 
 
+MAKERS = {"tudilix": hybrid_config, "llama": llama_config, "gikovik": gikovik_config, "mixtral": mixtral_config}
+PAIRS = {"tudilix": "llama", "gikovik": "mixtral"}
+
+
 def run(size: str = "2b", batch: int = 32, prompt_len: int = 1024, gen_len: int = 32, reps: int = 2,
         tmp: str = "/tmp/dllm_hybrid_bench", models=("tudilix", "llama")) -> dict:
+    """``models``: which to run, of tudilix, llama, gikovik, mixtral; a layer-list model and its flat
+    counterpart (tudilix / llama, gikovik / mixtral) also get the ratio of their throughputs."""
     out = {"size": size, "batch": batch, "prompt_len": prompt_len, "gen_len": gen_len, "dtype": "bf16",
            "data": "synthetic (random-init weights, random token ids)"}
-    for key, cfg, graphs in (("tudilix", hybrid_config(size), True), ("llama", llama_config(size), True)):
-        if key not in models:
-            continue
-        p, d = _measure(cfg, batch, prompt_len, gen_len, reps, f"{tmp}/{key}", graphs)
+    for key in models:
+        cfg = MAKERS[key](size)
+        p, d = _measure(cfg, batch, prompt_len, gen_len, reps, f"{tmp}/{key}", True)
         out[key] = {"prefill_tok_s": round(p, 1), "decode_tok_s": round(d, 1),
                     "params_m": round(cfg.param_count() / 1e6, 1)}
-    if len(models) < 2:
-        return out
-    out["prefill_ratio"] = round(out["tudilix"]["prefill_tok_s"] / out["llama"]["prefill_tok_s"], 3)
-    out["decode_ratio"] = round(out["tudilix"]["decode_tok_s"] / out["llama"]["decode_tok_s"], 3)
+    for a, b in PAIRS.items():
+        if a in out and b in out:
+            out["prefill_ratio"] = round(out[a]["prefill_tok_s"] / out[b]["prefill_tok_s"], 3)
+            out["decode_ratio"] = round(out[a]["decode_tok_s"] / out[b]["decode_tok_s"], 3)
     return out
