@@ -78,7 +78,7 @@ def latent_attention_sink(h, p, m, eps):
 
 
 def latent_attention_rot(h, p, m, eps):
-    """Latent attention with a rotated part: per head [dim unrotated | rot_dim rotated] queries, a
+    """Latent attention with a rotated part: queries of dim plain + rot_dim rotary dimensions per head, a
     single rotary key slice for every head (the last rot_dim rows of dkv, which skip the norm), per-head sigmoid
     output gate.  p: dq, dq.norm, uq, dkv, dkv.norm, uk, uv, g, o."""
     hn, d, dr, dv, r = m["heads"], m["dim"], m["rot_dim"], m["vdim"], m["kv_rank"]
