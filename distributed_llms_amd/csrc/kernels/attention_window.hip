@@ -642,12 +642,14 @@ static void launch_decode(uintptr_t out, uintptr_t q, uintptr_t k_cache, uintptr
                           int max_blocks, uintptr_t positions, uintptr_t tok_seq, int rows, int H, int G, int D,
                           int Dv, int bs, int window, float scale, uintptr_t sinks, int splits, uintptr_t ws,
                           uintptr_t stream) {
-  // heads per workgroup: 16 (all MFMA columns) when rows x K/V heads fill the chip, else halved until
-  // about half the CUs have a workgroup -- the keys are re-read from L2, the columns left idle cost nothing
+  // heads per workgroup: 16 (all MFMA columns) when rows x K/V heads x key runs fill the chip, else halved
+  // until about half the CUs have a workgroup -- the keys are re-read from L2, the columns left idle cost
+  // nothing.  Key runs come first: a workgroup holds a CU's registers alone, so the call takes
+  // (workgroups / CUs) rounds of one run's load chain, and head groups multiply the rounds, runs shorten them.
   const int R = H / G;
-  int hpw = std::min(16, R);
-  while (hpw > 2 && (long)rows * G * ((R + hpw - 1) / hpw) < 128) hpw = (hpw + 1) / 2;
   splits = ws ? std::max(1, std::min(splits, 64)) : 1;
+  int hpw = std::min(16, R);
+  while (hpw > 2 && (long)rows * G * ((R + hpw - 1) / hpw) * splits < 128) hpw = (hpw + 1) / 2;
   hipLaunchKernelGGL(HIP_KERNEL_NAME(window_attn_decode_kernel<NQK, NDV>),
                      dim3(rows, G * ((R + hpw - 1) / hpw), splits), dim3(64 * kDW), 0,
                      (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)k_cache, (const bf16*)v_cache,

@@ -52,12 +52,15 @@ PYBIND11_MODULE(_C_kernels, m) {
   m.def("lat_prep", &dllm::lat_prep);
   m.def("lat_q_pack", &dllm::lat_q_pack);
   m.def("lat_head_gate", &dllm::lat_head_gate);
+  m.def("lat_q_fold", &dllm::lat_q_fold);
+  m.def("lat_v_unfold", &dllm::lat_v_unfold);
   m.def("par_add", &dllm::par_add);
   m.def("stream_cat", &dllm::stream_cat);
   m.def("stream_set", &dllm::stream_set);
   m.def("side_gate", &dllm::side_gate);
   m.def("silu_glu", &dllm::silu_glu);
   m.def("moe_route_groups", &dllm::moe_route_groups);
+  m.def("moe_router_groups", &dllm::moe_router_groups);
   m.def("relu_sq", &dllm::relu_sq);
   m.def("moe_combine_gated", &dllm::moe_combine_gated);
   m.def("p2p_inbox_bytes", &dllm::p2p_inbox_bytes);

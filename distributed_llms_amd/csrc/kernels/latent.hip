@@ -155,6 +155,205 @@ void lat_q_pack(uintptr_t out, uintptr_t qa, uintptr_t q, int tokens, int H, int
                 (const int32_t*)positions);
 }
 
+// Few tokens (decode steps): the per-head products themselves, one workgroup per (token, head), instead
+// of a library batched product plus a pack / gate launch.
+//   lat_q_fold    q~[t, h] = [ q[t, h, :dim] . Wuk[h] ([dim, rank])  |  rotated q[t, h, dim:] ]
+//   lat_v_unfold  out[t, h] = (o_lat[t, h] . WuvT[h] ([rank, vdim])) * sigmoid(gate[t, h])
+// Consecutive threads own consecutive output columns, so every weight row is read in whole lines; the
+// token's vector sits in LDS as float; sums are float32.
+template <typename T>
+__global__ void __launch_bounds__(256) lat_q_fold_kernel(void* __restrict__ out_, const void* __restrict__ q_,
+                                                         const void* __restrict__ wuk_, int H, int rank, int dim,
+                                                         int rot_dim, const float* __restrict__ freqs, int nfreq,
+                                                         const int32_t* __restrict__ positions) {
+  extern __shared__ float qs[];                              // [dim]
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int D = rank + rot_dim, dq = dim + rot_dim;
+  T* out = (T*)out_ + ((size_t)t * H + h) * D;
+  const T* q = (const T*)q_ + ((size_t)t * H + h) * dq;
+  const T* w = (const T*)wuk_ + (size_t)h * dim * rank;
+  for (int d = threadIdx.x; d < dim; d += 256) qs[d] = ldf(q + d);
+  __syncthreads();
+  for (int j = threadIdx.x; j < rank; j += 256) {
+    float acc = 0.f;
+    for (int d = 0; d < dim; ++d) acc = fmaf(qs[d], ldf(w + (size_t)d * rank + j), acc);
+    stf(out + j, acc);
+  }
+  const float pos = (float)positions[t];
+  for (int i = threadIdx.x; i < (rot_dim + 1) / 2; i += 256) {
+    const T* qr = q + dim + 2 * i;
+    T* o = out + rank + 2 * i;
+    const float u = ldf(qr);
+    if (2 * i + 1 >= rot_dim) {
+      stf(o, u);
+      continue;
+    }
+    const float v = ldf(qr + 1);
+    float a = u, b = v;
+    if (i < nfreq) {
+      const float ang = pos * freqs[i];
+      const float c = cosf(ang), s = sinf(ang);
+      a = u * c - v * s;
+      b = v * c + u * s;
+    }
+    stf(o, a);
+    stf(o + 1, b);
+  }
+}
+
+// bf16 with 8 | rank: a thread owns 8 consecutive outputs (16-byte weight loads) and every ng-th input
+// row; the ng partial sums of an output meet in LDS.
+__global__ void __launch_bounds__(256) lat_q_fold_vec_kernel(bf16* __restrict__ out_, const bf16* __restrict__ q_,
+                                                             const bf16* __restrict__ wuk, int H, int rank, int dim,
+                                                             int rot_dim, const float* __restrict__ freqs, int nfreq,
+                                                             const int32_t* __restrict__ positions, int ng) {
+  extern __shared__ float sm[];
+  float* qs = sm;                                            // [dim]
+  float* red = sm + dim;                                     // [ng][rank]
+  const int t = blockIdx.x, h = blockIdx.y;
+  const int D = rank + rot_dim, dq = dim + rot_dim;
+  bf16* out = out_ + ((size_t)t * H + h) * D;
+  const bf16* q = q_ + ((size_t)t * H + h) * dq;
+  const bf16* w = wuk + (size_t)h * dim * rank;
+  for (int d = threadIdx.x; d < dim; d += 256) qs[d] = bf2f(q[d]);
+  __syncthreads();
+  const int nc = rank >> 3, c = threadIdx.x % nc, g = threadIdx.x / nc;
+  if (g < ng) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int d = g; d < dim; d += ng) {
+      const bf16x8 w8 = *reinterpret_cast<const bf16x8*>(w + (size_t)d * rank + 8 * c);
+      const float qv = qs[d];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(qv, bf2f(w8[i]), acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) red[g * rank + 8 * c + i] = acc[i];
+  }
+  __syncthreads();
+  for (int j = threadIdx.x; j < rank; j += 256) {
+    float s = 0.f;
+    for (int g2 = 0; g2 < ng; ++g2) s += red[g2 * rank + j];
+    out[j] = f2bf(s);
+  }
+  const float pos = (float)positions[t];
+  for (int i = threadIdx.x; i < (rot_dim + 1) / 2; i += 256) {
+    const bf16* qr = q + dim + 2 * i;
+    bf16* o = out + rank + 2 * i;
+    const float u = bf2f(qr[0]);
+    if (2 * i + 1 >= rot_dim) {
+      o[0] = f2bf(u);
+      continue;
+    }
+    const float v = bf2f(qr[1]);
+    float a = u, b = v;
+    if (i < nfreq) {
+      const float ang = pos * freqs[i];
+      const float cs = cosf(ang), sn = sinf(ang);
+      a = u * cs - v * sn;
+      b = v * cs + u * sn;
+    }
+    o[0] = f2bf(a);
+    o[1] = f2bf(b);
+  }
+}
+
+// groups of input rows for the vector forms: as many as 256 threads allow, at most one per input row
+static int fold_groups(int out_width, int in_width) { return std::max(1, std::min(256 / (out_width / 8), in_width)); }
+
+void lat_q_fold(uintptr_t out, uintptr_t q, uintptr_t wuk, int tokens, int H, int rank, int dim, int rot_dim,
+                uintptr_t freqs, int nfreq, uintptr_t positions, int f32, uintptr_t stream) {
+  if (tokens <= 0) return;
+  DLLM_HOST_CHECK(H > 0 && H <= 65535 && rank > 0 && dim > 0 && dim <= 8192 && rot_dim >= 0 && 2 * nfreq <= rot_dim,
+                  "latent query sizes");
+  DLLM_HOST_CHECK(out && q && wuk && (nfreq == 0 || freqs), "latent query arguments");
+  if (!f32 && rank % 8 == 0 && rank <= 2048) {
+    const int ng = fold_groups(rank, dim);
+    hipLaunchKernelGGL(lat_q_fold_vec_kernel, dim3(tokens, H), dim3(256), sizeof(float) * ((size_t)dim + (size_t)ng * rank),
+                       (hipStream_t)stream, (bf16*)out, (const bf16*)q, (const bf16*)wuk, H, rank, dim, rot_dim,
+                       (const float*)freqs, nfreq, (const int32_t*)positions, ng);
+    DLLM_HIP_CHECK(hipGetLastError());
+    return;
+  }
+  SM_DISPATCH(f32, lat_q_fold_kernel, dim3(tokens, H), dim3(256), sizeof(float) * dim, stream, (void*)out,
+              (const void*)q, (const void*)wuk, H, rank, dim, rot_dim, (const float*)freqs, nfreq,
+              (const int32_t*)positions);
+}
+
+template <typename T>
+__global__ void __launch_bounds__(256) lat_v_unfold_kernel(void* __restrict__ out_, const void* __restrict__ o_,
+                                                           const void* __restrict__ wuv_t_,
+                                                           const void* __restrict__ gate_, long ld, int H, int rank,
+                                                           int vdim) {
+  extern __shared__ float os[];                              // [rank]
+  const int t = blockIdx.x, h = blockIdx.y;
+  T* out = (T*)out_ + ((size_t)t * H + h) * vdim;
+  const T* o = (const T*)o_ + ((size_t)t * H + h) * rank;
+  const T* w = (const T*)wuv_t_ + (size_t)h * rank * vdim;
+  const T* gate = (const T*)gate_;
+  for (int r = threadIdx.x; r < rank; r += 256) os[r] = ldf(o + r);
+  __syncthreads();
+  const float g = gate ? 1.0f / (1.0f + expf(-ldf(gate + (size_t)t * ld + h))) : 1.0f;
+  for (int e = threadIdx.x; e < vdim; e += 256) {
+    float acc = 0.f;
+    for (int r = 0; r < rank; ++r) acc = fmaf(os[r], ldf(w + (size_t)r * vdim + e), acc);
+    // the product is rounded to the activation type before the gate, like the batched product it stands for
+    T y;
+    stf(&y, acc);
+    stf(out + e, ldf(&y) * g);
+  }
+}
+
+__global__ void __launch_bounds__(256) lat_v_unfold_vec_kernel(bf16* __restrict__ out_, const bf16* __restrict__ o_,
+                                                               const bf16* __restrict__ wuv_t,
+                                                               const bf16* __restrict__ gate, long ld, int H, int rank,
+                                                               int vdim, int ng) {
+  extern __shared__ float sm[];
+  float* os = sm;                                            // [rank]
+  float* red = sm + rank;                                    // [ng][vdim]
+  const int t = blockIdx.x, h = blockIdx.y;
+  bf16* out = out_ + ((size_t)t * H + h) * vdim;
+  const bf16* o = o_ + ((size_t)t * H + h) * rank;
+  const bf16* w = wuv_t + (size_t)h * rank * vdim;
+  for (int r = threadIdx.x; r < rank; r += 256) os[r] = bf2f(o[r]);
+  __syncthreads();
+  const int nc = vdim >> 3, c = threadIdx.x % nc, g = threadIdx.x / nc;
+  if (g < ng) {
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int r = g; r < rank; r += ng) {
+      const bf16x8 w8 = *reinterpret_cast<const bf16x8*>(w + (size_t)r * vdim + 8 * c);
+      const float ov = os[r];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) acc[i] = fmaf(ov, bf2f(w8[i]), acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) red[g * vdim + 8 * c + i] = acc[i];
+  }
+  __syncthreads();
+  const float gt = gate ? 1.0f / (1.0f + expf(-bf2f(gate[(size_t)t * ld + h]))) : 1.0f;
+  for (int e = threadIdx.x; e < vdim; e += 256) {
+    float s = 0.f;
+    for (int g2 = 0; g2 < ng; ++g2) s += red[g2 * vdim + e];
+    out[e] = f2bf(bf2f(f2bf(s)) * gt);           // rounded before the gate, like the batched product it stands for
+  }
+}
+
+void lat_v_unfold(uintptr_t out, uintptr_t o, uintptr_t wuv_t, uintptr_t gate, long ld, int tokens, int H, int rank,
+                  int vdim, int f32, uintptr_t stream) {
+  if (tokens <= 0) return;
+  DLLM_HOST_CHECK(H > 0 && H <= 65535 && rank > 0 && rank <= 8192 && vdim > 0 && out && o && wuv_t,
+                  "latent value arguments");
+  if (!f32 && vdim % 8 == 0 && vdim <= 2048) {
+    const int ng = fold_groups(vdim, rank);
+    hipLaunchKernelGGL(lat_v_unfold_vec_kernel, dim3(tokens, H), dim3(256),
+                       sizeof(float) * ((size_t)rank + (size_t)ng * vdim), (hipStream_t)stream, (bf16*)out,
+                       (const bf16*)o, (const bf16*)wuv_t, (const bf16*)gate, ld, H, rank, vdim, ng);
+    DLLM_HIP_CHECK(hipGetLastError());
+    return;
+  }
+  SM_DISPATCH(f32, lat_v_unfold_kernel, dim3(tokens, H), dim3(256), sizeof(float) * rank, stream, (void*)out,
+              (const void*)o, (const void*)wuv_t, (const void*)gate, ld, H, rank, vdim);
+}
+
 // out [T, H * vdim] = o [H, T, vdim] * sigmoid(gate[t * ld + h]) (gate null: a plain transposing copy);
 // one workgroup per (token, head)
 template <typename T, int V>

@@ -107,6 +107,10 @@ void lat_prep(uintptr_t cq, uintptr_t down, long ld, int q_off, int q_rank, uint
               uintptr_t stream);
 void lat_q_pack(uintptr_t out, uintptr_t qa, uintptr_t q, int tokens, int H, int rank, int dim, int rot_dim,
                 uintptr_t freqs, int nfreq, uintptr_t positions, int f32, uintptr_t stream);
+void lat_q_fold(uintptr_t out, uintptr_t q, uintptr_t wuk, int tokens, int H, int rank, int dim, int rot_dim,
+                uintptr_t freqs, int nfreq, uintptr_t positions, int f32, uintptr_t stream);
+void lat_v_unfold(uintptr_t out, uintptr_t o, uintptr_t wuv_t, uintptr_t gate, long ld, int tokens, int H, int rank,
+                  int vdim, int f32, uintptr_t stream);
 void lat_head_gate(uintptr_t out, uintptr_t o, uintptr_t gate, long ld, int tokens, int H, int vdim, int f32,
                    uintptr_t stream);
 void par_add(uintptr_t x, uintptr_t a, uintptr_t b, uintptr_t x_rounded, long n, int f32, uintptr_t stream);
@@ -119,6 +123,9 @@ void side_gate(uintptr_t g, uintptr_t z, uintptr_t table, uintptr_t ids, int tok
 void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, int E, int k, int groups, int keep,
                       float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts, uintptr_t offsets,
                       uintptr_t sorted_tok, uintptr_t inv, uintptr_t stream);
+void moe_router_groups(uintptr_t x, uintptr_t w, int K, int rows, uintptr_t logits, uintptr_t correction, int T, int E,
+                       int k, int groups, int keep, float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts,
+                       uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, int f32, uintptr_t stream);
 void relu_sq(uintptr_t y, long n, int f32, uintptr_t stream);
 void moe_combine_gated(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t inv, uintptr_t shared,
                        uintptr_t gate_logits, long gate_ld, int T, int H, int k, int f32, uintptr_t stream);

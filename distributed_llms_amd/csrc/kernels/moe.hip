@@ -377,16 +377,15 @@ void moe_combine(uintptr_t out, uintptr_t ysorted, uintptr_t topk_w, uintptr_t i
 constexpr int kMaxGroups = 64;
 constexpr int kMaxChoiceExperts = 256;
 
+// one token's selection from its E logits `lg`
 template <int EMAX>
-__global__ void __launch_bounds__(128) moe_choice_groups_kernel(
-    const float* __restrict__ logits, long ld, const float* __restrict__ correction, int T, int E, int k, int groups,
-    int keep, float scale, float* __restrict__ topk_w, int* __restrict__ topk_ids) {
-  const int t = blockIdx.x * 128 + threadIdx.x;
-  if (t >= T) return;
+__device__ __forceinline__ void choose_groups(const float* __restrict__ lg, const float* __restrict__ correction, int E,
+                                              int k, int groups, int keep, float scale, float* __restrict__ tw,
+                                              int* __restrict__ ti) {
   const int gsz = E / groups;
   float sc[EMAX], ch[EMAX];
   for (int e = 0; e < E; ++e) {
-    sc[e] = 1.0f / (1.0f + expf(-logits[(size_t)t * ld + e]));
+    sc[e] = 1.0f / (1.0f + expf(-lg[e]));
     ch[e] = sc[e] + (correction ? correction[e] : 0.f);
   }
   if (keep < groups) {
@@ -425,9 +424,55 @@ __global__ void __launch_bounds__(128) moe_choice_groups_kernel(
     tot += sc[best];
   }
   for (int j = 0; j < k; ++j) {
-    topk_ids[t * k + j] = ids[j];
-    topk_w[t * k + j] = sc[ids[j]] / (tot + 1e-20f) * scale;
+    ti[j] = ids[j];
+    tw[j] = sc[ids[j]] / (tot + 1e-20f) * scale;
   }
+}
+
+template <int EMAX>
+__global__ void __launch_bounds__(128) moe_choice_groups_kernel(
+    const float* __restrict__ logits, long ld, const float* __restrict__ correction, int T, int E, int k, int groups,
+    int keep, float scale, float* __restrict__ topk_w, int* __restrict__ topk_ids) {
+  const int t = blockIdx.x * 128 + threadIdx.x;
+  if (t >= T) return;
+  choose_groups<EMAX>(logits + (size_t)t * ld, correction, E, k, groups, keep, scale, topk_w + (size_t)t * k,
+                      topk_ids + (size_t)t * k);
+}
+
+// Few tokens (decode steps): the router product and the selection in one launch, a workgroup per token.
+// x [T, K] (bf16 or float) times the float32 rows w [rows, K] (the E router rows, then any further rows
+// such as a shared expert's gate), float32 sums, written to logits [T, rows]; then one thread selects.
+template <typename TX, int EMAX>
+__global__ void __launch_bounds__(256) moe_router_groups_kernel(
+    const TX* __restrict__ x, const float* __restrict__ w, int K, int rows, float* __restrict__ logits,
+    const float* __restrict__ correction, int E, int k, int groups, int keep, float scale, float* __restrict__ topk_w,
+    int* __restrict__ topk_ids) {
+  __shared__ float lg[kMaxChoiceExperts + 8];
+  const int t = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+  const TX* xr = x + (size_t)t * K;
+  for (int r = wv; r < rows; r += 4) {
+    const float* wr = w + (size_t)r * K;
+    float acc = 0.f;
+    if ((K & 7) == 0) {                            // 8 elements per lane and step: 16- and 32-byte loads
+      for (int c = lane * 8; c < K; c += 512) {
+        float xv[8], wv8[8];
+        ldv<8>(xr + c, xv);
+        ldv<8>(wr + c, wv8);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc = fmaf(xv[i], wv8[i], acc);
+      }
+    } else {
+      for (int c = lane; c < K; c += 64) acc = fmaf((float)xr[c], wr[c], acc);
+    }
+    acc = wave_sum(acc);
+    if (lane == 0) {
+      lg[r] = acc;
+      logits[(size_t)t * rows + r] = acc;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x == 0)
+    choose_groups<EMAX>(lg, correction, E, k, groups, keep, scale, topk_w + (size_t)t * k, topk_ids + (size_t)t * k);
 }
 
 __global__ void __launch_bounds__(1024) moe_scatter_wide_kernel(const int* __restrict__ topk_ids, int T, int E, int k,
@@ -473,6 +518,30 @@ void moe_route_groups(uintptr_t logits, long ld, uintptr_t correction, int T, in
   else if (E <= 64) ROUTE_G(64);
   else ROUTE_G(256);
 #undef ROUTE_G
+  DLLM_HIP_CHECK(hipGetLastError());
+  hipLaunchKernelGGL(moe_scatter_wide_kernel, dim3(1), dim3(1024), 0, s, (const int*)topk_ids, T, E, k, (int*)counts,
+                     (int*)offsets, (int*)sorted_tok, (int*)inv);
+  DLLM_HIP_CHECK(hipGetLastError());
+}
+
+void moe_router_groups(uintptr_t x, uintptr_t w, int K, int rows, uintptr_t logits, uintptr_t correction, int T, int E,
+                       int k, int groups, int keep, float scale, uintptr_t topk_w, uintptr_t topk_ids, uintptr_t counts,
+                       uintptr_t offsets, uintptr_t sorted_tok, uintptr_t inv, int f32, uintptr_t stream) {
+  DLLM_HOST_CHECK(E >= 1 && E <= kMaxChoiceExperts && rows >= E && rows <= kMaxChoiceExperts + 8 && K > 0,
+                  "1 <= experts <= 256, up to 8 further rows");
+  DLLM_HOST_CHECK(k >= 1 && k <= 16 && k <= E, "1 <= top <= min(16, experts)");
+  DLLM_HOST_CHECK(groups >= 1 && groups <= kMaxGroups && E % groups == 0 && keep >= 1 && keep <= groups &&
+                      keep * (E / groups) >= k,
+                  "expert groups");
+  if (T <= 0) return;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+#define ROUTER_G(TX, EMAX)                                                                                       \
+  hipLaunchKernelGGL((moe_router_groups_kernel<TX, EMAX>), dim3(T), dim3(256), 0, s, (const TX*)x, (const float*)w, \
+                     K, rows, (float*)logits, (const float*)correction, E, k, groups, keep, scale, (float*)topk_w,  \
+                     (int*)topk_ids)
+  if (f32) { if (E <= 16) ROUTER_G(float, 16); else if (E <= 64) ROUTER_G(float, 64); else ROUTER_G(float, 256); }
+  else { if (E <= 16) ROUTER_G(bf16, 16); else if (E <= 64) ROUTER_G(bf16, 64); else ROUTER_G(bf16, 256); }
+#undef ROUTER_G
   DLLM_HIP_CHECK(hipGetLastError());
   hipLaunchKernelGGL(moe_scatter_wide_kernel, dim3(1), dim3(1024), 0, s, (const int*)topk_ids, T, E, k, (int*)counts,
                      (int*)offsets, (int*)sorted_tok, (int*)inv);

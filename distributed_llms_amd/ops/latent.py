@@ -25,6 +25,9 @@ from . import seqmix as sm
 from .seqmix import SeqBatch, _ck, _f32flag, _k, _ptr, _stream
 
 
+FOLD_MAX_TOKENS = 64      # up to this many tokens the per-head products run in the fold / unfold kernels
+
+
 @dataclass
 class LatentSpec:
     """Sizes and constants of one latent-attention mixer."""
@@ -94,9 +97,17 @@ def latent_queries(q: torch.Tensor, w_uk: torch.Tensor, spec: LatentSpec, freqs:
     ``w_uk`` [H, dim, rank] (the key up-projection folded into the query) next to the rotated part."""
     t = q.shape[0]
     h, d, dr, r = spec.heads, spec.dim, spec.rot_dim, spec.rank
+    nf = 0 if freqs is None else freqs.numel()
+    if q.is_cuda and t <= FOLD_MAX_TOKENS:
+        # few tokens: product, rotation and concatenation in one launch
+        _ck(q, "q")
+        _ck(w_uk, "w_uk", q.dtype)
+        out = torch.empty(t, h, r + dr, dtype=q.dtype, device=q.device)
+        _k().lat_q_fold(out.data_ptr(), q.data_ptr(), w_uk.data_ptr(), t, h, r, d, dr, _ptr(freqs), nf,
+                        positions.data_ptr(), _f32flag(q), _stream())
+        return out
     q3 = q.view(t, h, d + dr)
     qa = torch.bmm(q3[:, :, :d].transpose(0, 1), w_uk)                    # [H, T, rank]
-    nf = 0 if freqs is None else freqs.numel()
     if not q.is_cuda:
         parts = [qa.transpose(0, 1)]
         if dr:
@@ -115,8 +126,19 @@ def latent_values(o_lat: torch.Tensor, w_uv_t: torch.Tensor, gate: Optional[torc
     """o_lat [T, H, rank] (softmax-weighted sums of latents) -> [T, H * vdim]: per head times
     ``w_uv_t`` [H, rank, vdim], then times sigmoid(gate[t, gate_col + h]) when ``gate`` (a [T, *] tensor
     holding one gate logit per head from column ``gate_col``) is given."""
-    t, h, _ = o_lat.shape
+    t, h, r = o_lat.shape
     vd = w_uv_t.shape[2]
+    if o_lat.is_cuda and t <= FOLD_MAX_TOKENS:
+        # few tokens: product, gate and the [T, H vdim] layout in one launch
+        _ck(o_lat, "o_lat")
+        _ck(w_uv_t, "w_uv_t", o_lat.dtype)
+        if gate is not None:
+            _ck(gate, "gate", o_lat.dtype)
+        out = torch.empty(t, h * vd, dtype=o_lat.dtype, device=o_lat.device)
+        gp = 0 if gate is None else gate.data_ptr() + gate_col * gate.element_size()
+        _k().lat_v_unfold(out.data_ptr(), o_lat.data_ptr(), w_uv_t.data_ptr(), gp, 0 if gate is None else gate.shape[1],
+                          t, h, r, vd, _f32flag(o_lat), _stream())
+        return out
     o = torch.bmm(o_lat.transpose(0, 1), w_uv_t)                          # [H, T, vdim]
     if not o_lat.is_cuda:
         o = o.transpose(0, 1).float()

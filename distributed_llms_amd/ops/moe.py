@@ -24,6 +24,7 @@ from .. import _ext, knobs
 from . import reference as ref
 
 GROUPED_MAX_TOKENS = 256      # beyond this the per-expert row count makes library GEMMs cheaper
+ROUTER_FUSED_MAX_TOKENS = 64  # up to this many tokens the grouped-choice router product runs inside the selection kernel
 # knobs.moe_variant: 0 = pick by expected rows per expert; 1..6 force a kernel variant
 # (bench/moe_bench.py sweeps them).  knobs.moe_wide_min_pairs: token-expert pairs (T x top_k) from
 # which the MFMA-tiled grouped kernel (gemm_wide.hip moe_wide_gemm) replaces the weight-streaming
@@ -182,8 +183,8 @@ def grouped_choice_ffn(x: torch.Tensor, w_router: torch.Tensor, correction: Opti
     has_shared = shared_up is not None
     if w_router.shape[0] != e + (1 if has_shared else 0) or w_router.dtype != torch.float32:
         raise ValueError("grouped_choice_ffn: router rows = experts (+ 1 with a shared expert), float32")
-    logits = F.linear(x.float(), w_router)                       # float32 also for bf16 activations
     if not x.is_cuda:
+        logits = F.linear(x.float(), w_router)                   # float32 also for bf16 activations
         tw, ids = route_grouped_choice(logits, correction, e, top, groups, keep, scale)
         out = torch.zeros(t, width, dtype=torch.float32)
         xf = x.float()
@@ -201,7 +202,7 @@ def grouped_choice_ffn(x: torch.Tensor, w_router: torch.Tensor, correction: Opti
     st = torch.cuda.current_stream().cuda_stream
     dev = x.device
     f32 = 1 if x.dtype == torch.float32 else 0
-    if not (x.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous() and logits.is_contiguous()):
+    if not (x.is_contiguous() and w_up.is_contiguous() and w_down.is_contiguous() and w_router.is_contiguous()):
         raise ValueError("grouped_choice_ffn: operands must be contiguous")
     if correction is not None and (correction.dtype != torch.float32 or correction.numel() != e):
         raise ValueError("grouped_choice_ffn: correction is float32 [E]")
@@ -211,14 +212,33 @@ def grouped_choice_ffn(x: torch.Tensor, w_router: torch.Tensor, correction: Opti
     offsets = torch.empty(e + 1, dtype=torch.int32, device=dev)
     sorted_tok = torch.empty(t * top, dtype=torch.int32, device=dev)
     inv = torch.empty(t * top, dtype=torch.int32, device=dev)
-    k.moe_route_groups(logits.data_ptr(), logits.shape[1], 0 if correction is None else correction.data_ptr(), t, e,
-                       top, groups, keep, float(scale), topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(),
-                       offsets.data_ptr(), sorted_tok.data_ptr(), inv.data_ptr(), st)
+    cp = 0 if correction is None else correction.data_ptr()
+    if t <= ROUTER_FUSED_MAX_TOKENS:
+        # few tokens: the float32 router product and the selection in one launch (+ the scatter)
+        logits = torch.empty(t, w_router.shape[0], dtype=torch.float32, device=dev)
+        k.moe_router_groups(x.data_ptr(), w_router.data_ptr(), width, w_router.shape[0], logits.data_ptr(), cp, t, e, top,
+                            groups, keep, float(scale), topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(),
+                            offsets.data_ptr(), sorted_tok.data_ptr(), inv.data_ptr(), f32, st)
+    else:
+        logits = F.linear(x.float(), w_router)                   # float32 also for bf16 activations
+        k.moe_route_groups(logits.data_ptr(), logits.shape[1], cp, t, e, top, groups, keep, float(scale),
+                           topk_w.data_ptr(), topk_ids.data_ptr(), counts.data_ptr(), offsets.data_ptr(),
+                           sorted_tok.data_ptr(), inv.data_ptr(), st)
     slots = t * top
     ys = torch.empty(slots, width, dtype=x.dtype, device=dev)
     bf = x.dtype == torch.bfloat16
-    if bf and t <= GROUPED_MAX_TOKENS and width % 128 == 0 and f % 128 == 0:
-        # decode-sized: grouped weight-streaming GEMMs on the expert-sorted slots, no host sync
+    if bf and t <= GROUPED_MAX_TOKENS and width % 128 == 0 and f % 128 == 0 and 0 < knobs.K.moe_wide_min_pairs <= slots:
+        # decode-sized with several rows per expert: the MFMA-tiled grouped kernel (it has no squared-ReLU
+        # epilogue: the activation is a launch of its own on the small [slots, F] tensor), no host sync
+        act = torch.empty(slots, f, dtype=x.dtype, device=dev)
+        ring = 0 if knobs.K.moe_deep_ring else 4
+        k.moe_wide_gemm(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_up.data_ptr(), counts.data_ptr(),
+                        offsets.data_ptr(), e, f, width, ring, st)
+        k.relu_sq(act.data_ptr(), act.numel(), 0, st)
+        k.moe_wide_gemm(ys.data_ptr(), act.data_ptr(), 0, w_down.data_ptr(), counts.data_ptr(), offsets.data_ptr(), e,
+                        width, f, ring, st)
+    elif bf and t <= GROUPED_MAX_TOKENS and width % 128 == 0 and f % 128 == 0:
+        # a few rows: grouped weight-streaming GEMMs on the expert-sorted slots, no host sync
         act = torch.empty(slots, f, dtype=x.dtype, device=dev)
         rows = -(-slots // e)
         k.moe_grouped_gemm(act.data_ptr(), x.data_ptr(), sorted_tok.data_ptr(), w_up.data_ptr(), counts.data_ptr(),
